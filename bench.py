@@ -1,0 +1,334 @@
+#!/usr/bin/env python3
+"""bench.py -- reduce+codec throughput of one 25 MiB DDP bucket on one MI355X.
+
+A "step" is one pass of the hot path over one bucket: the fused
+bf16-decode + reduce + average fold of configuration C2 (butterfly schedule,
+3 virtual ranks, 6,553,600 fp32 gradients per rank, bf16 wire, x 1/3) -- every
+virtual rank folds its own chunk of the bucket from its own fp32 data and the
+two peers' bf16 wire chunks, all resident in HBM, in ONE launch.
+
+Algorithmic bytes per step (what `value` and `roofline.achieved` are computed
+from): per bucket element 4 B own fp32 read + 2 x 2 B bf16 peer reads + 4 B fp32
+write = 12 B  ->  78,643,200 B.
+
+The K timed steps are recorded into one HIP graph and replayed with a single
+submission, so the host's launch cost is not part of the measurement; steps
+rotate over several distinct copies of the workload (> 512 MiB in total) so the
+256 MiB Infinity Cache cannot serve the reads ("cold", the headline); the same
+loop over one copy is reported as "warm".
+
+Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--sets", type=int, default=8, help="distinct workload copies the cold loop rotates over")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="headline only (used when profiling)")
+    ap.add_argument("--no-cpu", action="store_true")
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU's share of the path; this build runs on a single GPU "
+              "(--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from mccl_amd import _lib as L
+    from mccl_amd import kernels as K
+    from mccl_amd import harness as H
+    from mccl_amd import workloads as W
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    q = K.ReduceQueue(0)
+    cfg = W.C2
+    world, numel = cfg["world"], cfg["numel"]
+    chunks = H.chunkize(numel, 1, world)
+    scale = 1.0 / world
+    bytes_per_step = numel * 12
+
+    # ---- workload: `sets` copies of (3 fp32 rank tensors + their bf16 wire copies)
+    host0 = [W.c2_input(r) for r in range(world)]
+    tensors, wires = [], []
+    for s in range(args.sets):
+        ts = [torch.from_numpy(host0[r]).cuda() if s == 0 else
+              torch.from_numpy(W.c2_input(r, variant=s)).cuda() for r in range(world)]
+        ws = [K.encode_bf16(t, queue=q) for t in ts]
+        tensors.append(ts)
+        wires.append(ws)
+    q.drain()
+
+    plan = K.make_plan(L.BF16, world, io=L.IO_OWN_FIRST_F32, op=L.SUM, scale_mode=L.SCALE_VIEW, scale=scale)
+
+    def step_segs(s, with_wire_out=False, out_tensors=None):
+        segs = []
+        for R, (start, cnt, _, _) in enumerate(chunks):
+            own = tensors[s][R].data_ptr() + start * 4
+            out = own if out_tensors is None else out_tensors[R].data_ptr() + start * 4
+            peers = [wires[s][p].data_ptr() + start * 2 for p in range(world) if p != R]
+            wire_out = wires[s][R].data_ptr() + start * 2 if with_wire_out else 0
+            segs.append(K.make_seg(out, wire_out, [own] + peers, cnt))
+        return segs
+
+    # ---- parity of exactly this launch against the CPU oracle (set 0, out of place)
+    from oracle import oracle as orc
+    outs = [torch.zeros_like(t) for t in tensors[0]]
+    q.fold(plan, step_segs(0, out_tensors=outs))
+    q.drain()
+    wire_host = [orc.encode_bf16(x) for x in host0]
+    parity = True
+    for R, (start, cnt, _, _) in enumerate(chunks):
+        peers = [np.ascontiguousarray(wire_host[p][start:start + cnt]) for p in range(world) if p != R]
+        want = orc.wire_fold_chunk(np.ascontiguousarray(host0[R][start:start + cnt]), peers,
+                                   scale_by=scale, threads=min(16, orc.max_threads()))
+        got = outs[R][start:start + cnt].cpu().numpy()
+        parity &= bool(np.array_equal(got.view(np.uint32), want.view(np.uint32)))
+    del outs
+
+    # ---- timed loops, each recorded into one graph
+    def record(n_steps, seg_fn):
+        q.graph_begin()
+        for i in range(n_steps):
+            seg_fn(i)
+        return q.graph_end()
+
+    def timed(graph):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        q.timer_begin()
+        q.graph_launch(graph)
+        ms_dev = q.timer_end()
+        torch.cuda.synchronize()
+        return ms_dev, (time.perf_counter() - t0) * 1e3
+
+    def measure(seg_fn, steps, warmup):
+        gw = record(max(1, warmup), seg_fn)
+        gk = record(steps, seg_fn)
+        q.graph_launch(gw)
+        q.drain()
+        ms_dev, ms_wall = timed(gk)
+        q.graph_destroy(gw)
+        q.graph_destroy(gk)
+        return ms_dev, ms_wall
+
+    cold = lambda i: q.fold(plan, step_segs(i % args.sets))
+    warm = lambda i: q.fold(plan, step_segs(0))
+    cold_dev, cold_wall = measure(cold, args.steps, args.warmup)
+    warm_dev, _ = measure(warm, args.steps, args.warmup)
+
+    gbs = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
+    kernel_us = cold_dev / args.steps * 1e3
+    achieved = gbs(bytes_per_step, cold_dev / args.steps)
+    value = gbs(bytes_per_step * args.steps, cold_wall)
+
+    result = {
+        "metric": "reduce+codec GB/s per 25 MB bucket and % of HBM peak, 1 MI355X vs host CPU",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(cold_wall / args.steps, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "C2: butterfly schedule, 3 virtual ranks, 6,553,600 fp32 grads (25 MiB) per rank, "
+                               "bf16 RNE wire, fused decode+accumulate+x(1/3), peers HBM-resident, "
+                               f"cold (rotating {args.sets} copies)",
+                   "algorithmic_bytes_per_step": bytes_per_step, "parity_vs_oracle_bit_exact": parity},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "fold_few_kernel<bf16, own-first fp32, k=3>", "kernel_us": round(kernel_us, 2)},
+    }
+    extra = {"warm_GBps": round(gbs(bytes_per_step, warm_dev / args.steps), 1),
+             "warm_kernel_us": round(warm_dev / args.steps * 1e3, 2),
+             "pct_of_hbm_peak_cold": round(100 * achieved / HBM_PEAK_GBS, 2)}
+
+    if not args.no_extras:
+        try:
+            extra.update(extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_segs,
+                                measure, gbs))
+        except Exception as e:  # extras never take the headline down
+            extra["extras_error"] = f"{type(e).__name__}: {e}"
+
+    # ---- CPU baseline: the same job in reference-shaped passes on the host cores
+    if not args.no_cpu:
+        threads = min(16, orc.max_threads())
+        own = [np.ascontiguousarray(host0[R][s:s + c]) for R, (s, c, _, _) in enumerate(chunks)]
+        prs = [[np.ascontiguousarray(wire_host[p][s:s + c]) for p in range(world) if p != R]
+               for R, (s, c, _, _) in enumerate(chunks)]
+
+        def cpu_pass(th):
+            t0 = time.perf_counter()
+            for R in range(world):
+                orc.wire_fold_chunk(own[R], prs[R], scale_by=scale, threads=th)
+            return time.perf_counter() - t0
+
+        def best_of(th, budget):
+            cpu_pass(th)
+            best, spent, reps = 1e9, 0.0, 0
+            while spent < budget and reps < 200:
+                dt = cpu_pass(th)
+                best, spent, reps = min(best, dt), spent + dt, reps + 1
+            return best, reps
+
+        b_all, reps_all = best_of(threads, args.cpu_seconds * 0.6)
+        b_one, reps_one = best_of(1, args.cpu_seconds * 0.4)
+        result["cpu_baseline"] = {
+            "value": round(bytes_per_step / b_all / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"the same C2 bucket (3 chunks, 78,643,200 algorithmic bytes) as reference-shaped passes "
+                      f"(encode, 2 binary bf16 reduces, scale, decode); best of {reps_all} passes, OpenMP",
+            "single_thread_GBps": round(bytes_per_step / b_one / 1e9, 2), "host_cpus": os.cpu_count()}
+    result["extra"] = extra
+    print(json.dumps(result))
+
+
+def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_segs, measure, gbs):
+    """Secondary measurements: the other legs of C2 and the other configurations."""
+    out = {}
+    world, numel = 3, W.C2["numel"]
+    sets = len(tensors)
+    steps, warm = max(20, args.steps // 4), 5
+
+    # C2 with the bf16 wire copy for the allgather leg also written (14 B/elem)
+    ms, _ = measure(lambda i: q.fold(plan, step_segs(i % sets, with_wire_out=True)), steps, warm)
+    out["c2_fold_with_wire_out_GBps"] = round(gbs(numel * 14, ms / steps), 1)
+
+    # encode leg: 3 ranks x (4 B read + 2 B write) per element
+    def enc(i):
+        s = i % sets
+        q.fold(K.make_plan(L.BF16, 1, io=L.IO_OWN_FIRST_F32),
+               [K.make_seg(0, wires[s][r].data_ptr(), [tensors[s][r].data_ptr()], numel) for r in range(world)])
+    ms, _ = measure(enc, steps, warm)
+    out["c2_encode_GBps"] = round(gbs(world * numel * 6, ms / steps), 1)
+
+    # whole allreduce of the bucket for all 3 virtual ranks: fused vs the reference's launch sequence
+    ws = H.Workspace(q, 3 * (numel * 2 + 256) + 3 * (2 * ((numel + 2) // 3) * 2 + 256))
+    for mode, name in ((L.REPLAY_FUSED, "fused"), (L.REPLAY_STEPWISE, "stepwise")):
+        def rep(i, mode=mode):
+            H.allreduce_replay(tensors[i % sets], "avg", L.ALGO_BUTTERFLY, wire_bf16=True, mode=mode,
+                               queue=q, workspace=ws, sync=False)
+        q.drain()
+        # cross-stream waits cannot be recorded: time these eagerly
+        for i in range(warm):
+            rep(i)
+        q.drain()
+        q.timer_begin()
+        for i in range(steps):
+            rep(i)
+        ms = q.timer_end()
+        out[f"c2_allreduce_{name}_us_per_bucket"] = round(ms / steps * 1e3, 1)
+    ws.free()
+
+    # C1: ring, 2 ranks, 1 Mi fp32, SUM: one k=2 fold per chunk
+    x = [torch.randn(W.C1["numel"], device="cuda") for _ in range(2 * 8)]
+    c1 = H.chunkize(W.C1["numel"], 1, 2)
+
+    def c1_step(i):
+        a, b = x[2 * (i % 8)], x[2 * (i % 8) + 1]
+        segs = []
+        for ch, (s, c, _, _) in enumerate(c1):
+            owner = (a, b)[(ch - 1) % 2]
+            first, last = (a, b)[ch], (a, b)[(ch + 1) % 2]
+            segs.append(K.make_seg(owner.data_ptr() + 4 * s, 0, [first.data_ptr() + 4 * s, last.data_ptr() + 4 * s], c))
+        q.fold(K.make_plan(L.F32, 2), segs)
+    ms, _ = measure(c1_step, steps, warm)
+    out["c1_ring_fold_us"] = round(ms / steps * 1e3, 2)
+    out["c1_ring_fold_GBps"] = round(gbs(12_582_912, ms / steps), 1)
+    del x
+
+    # C4: 4096 x 64 KiB messages x 3 ranks, one persistent table launch
+    n4, m4 = W.C4["numel"], W.C4["messages"]
+    r4 = [torch.rand(n4 * m4, device="cuda") * 2 - 1 for _ in range(3)]
+    segs4 = [K.make_seg(r4[0].data_ptr() + 4 * n4 * m, 0, [t.data_ptr() + 4 * n4 * m for t in r4], n4)
+             for m in range(m4)]
+    p4 = K.make_plan(L.F32, 3, topo=L.TOPO_BINOMIAL)
+    ms, _ = measure(lambda i: q.fold(p4, segs4), 10, 2)
+    out["c4_tree_batched_us_total"] = round(ms / 10 * 1e3, 1)
+    out["c4_tree_batched_ns_per_message"] = round(ms / 10 * 1e6 / m4, 1)
+    out["c4_tree_batched_GBps"] = round(gbs(4 * 65536 * m4, ms / 10), 1)
+    del r4, segs4
+
+    # C3: ring, 4 ranks, 110,000,002 fp32, bf16 wire, own operand last; peers in HBM, then in pinned host memory
+    n3 = W.C3["numel"]
+    c3 = H.chunkize(n3, 1, 4)
+    t3 = [torch.randn(n3, device="cuda") * 1e-4 for _ in range(4)]
+    w3 = [K.encode_bf16(t, queue=q) for t in t3]
+    q.drain()
+    p3 = K.make_plan(L.BF16, 4, io=L.IO_OWN_LAST_F32)
+
+    def c3_segs(wire_ptr):
+        segs = []
+        for ch, (s, c, _, _) in enumerate(c3):
+            o = (ch - 1) % 4
+            ins = [wire_ptr[(ch + j) % 4] + 2 * s for j in range(3)] + [t3[o].data_ptr() + 4 * s]
+            segs.append(K.make_seg(t3[o].data_ptr() + 4 * s, 0, ins, c))
+        return segs
+    hbm_segs = c3_segs([w.data_ptr() for w in w3])
+    ms, _ = measure(lambda i: q.fold(p3, hbm_segs), 10, 2)
+    out["c3_ring_fold_hbm_us"] = round(ms / 10 * 1e3, 1)
+    out["c3_ring_fold_hbm_GBps"] = round(gbs(n3 * 14, ms / 10), 1)
+    host_bufs = []
+    try:
+        dev_ptrs = []
+        for w in w3:
+            hptr, dptr = q.host_alloc(n3 * 2)
+            host_bufs.append(hptr)
+            dev_ptrs.append(dptr)
+            q.copy(dptr, w.data_ptr(), n3 * 2)
+        q.drain()
+        pin_segs = c3_segs(dev_ptrs)
+        ms, _ = measure(lambda i: q.fold(p3, pin_segs), 3, 1)
+        out["c3_ring_fold_pinned_host_ms"] = round(ms / 3, 2)
+        out["c3_ring_fold_pinned_host_PCIe_GBps"] = round(gbs(n3 * 6, ms / 3), 1)
+    finally:
+        for hptr in host_bufs:
+            q.host_free(hptr)
+    del t3, w3
+
+    # C5: reduce_scatter (8-input bf16 fold per rank, per-step rounding) and the allgather copy
+    n5, w5 = W.C5["numel"], 8
+    ch5 = n5 // w5
+    i5 = [(torch.randn(n5, device="cuda") * 1e-2).to(torch.bfloat16) for _ in range(w5)]
+    o5 = [torch.empty(ch5, dtype=torch.bfloat16, device="cuda") for _ in range(w5)]
+    for acc, name in ((L.ACC_STEP, "ref_exact"), (L.ACC_F32, "f32acc")):
+        p5 = K.make_plan(L.BF16, w5, acc=acc)
+        segs5 = [K.make_seg(o5[r].data_ptr(), 0,
+                            [i5[r].data_ptr() + 2 * ch5 * r] + [i5[p].data_ptr() + 2 * ch5 * r for p in range(w5) if p != r],
+                            ch5) for r in range(w5)]
+        ms, _ = measure(lambda i: q.fold(p5, segs5), 5, 1)
+        out[f"c5_reduce_scatter_{name}_us"] = round(ms / 5 * 1e3, 1)
+        out[f"c5_reduce_scatter_{name}_GBps"] = round(gbs(9 * ch5 * 2 * w5, ms / 5), 1)
+    g5 = torch.empty(n5, dtype=torch.bfloat16, device="cuda")
+    ms, _ = measure(lambda i: [q.copy(g5.data_ptr() + 2 * ch5 * p, o5[p].data_ptr(), 2 * ch5) for p in range(w5)], 5, 1)
+    out["c5_allgather_copy_one_rank_GBps"] = round(gbs(2 * n5 * 2, ms / 5), 1)
+    return out
+
+
+if __name__ == "__main__":
+    main()

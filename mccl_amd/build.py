@@ -1,0 +1,87 @@
+"""Compiles libmcclx.so (HIP kernels + C ABI + chunk scheduler) for gfx950.
+
+hipcc cross-compiles without a GPU.  The shared library is written next to this
+file so that it travels with the source tree; objects go to build/.
+
+    python -m mccl_amd.build            # build if sources are newer than the library
+    python -m mccl_amd.build --force
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+OBJ_DIR = os.path.join(ROOT, "build", "mcclx")
+LIB_PATH = os.path.join(HERE, "libmcclx.so")
+
+SOURCES = ["fold_kernels.hip", "copy_kernel.hip", "mcclx_api.cpp", "mcclx_sched.cpp"]
+HEADERS = ["fold_launch.h", "mcclx_internal.h", os.path.join(ROOT, "include", "mcclx.h")]
+
+# -ffp-contract=off / -fno-fast-math: IEEE fp32 add and mul, no FMA fusion, so
+# the kernels match the CPU oracle bit for bit.  Denormals are kept (hipcc's
+# default for gfx9).  Packed-FP32 instructions are disabled.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",
+    "-fno-gpu-flush-denormals-to-zero",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-fvisibility=hidden", "-Wall", "-Wno-unused-command-line-argument",
+    "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+]
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found: libmcclx.so cannot be built")
+    return exe
+
+
+def _newest_source_mtime() -> float:
+    paths = [os.path.join(CSRC, s) for s in SOURCES]
+    paths += [h if os.path.isabs(h) else os.path.join(CSRC, h) for h in HEADERS]
+    return max(os.path.getmtime(p) for p in paths)
+
+
+def needs_build() -> bool:
+    return not os.path.exists(LIB_PATH) or os.path.getmtime(LIB_PATH) < _newest_source_mtime()
+
+
+def build(force: bool = True, verbose: bool = False) -> str:
+    """Compile every source and link mccl_amd/libmcclx.so.  Returns its path."""
+    if not force and not needs_build():
+        return LIB_PATH
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    cc = hipcc()
+    procs = []
+    objs = []
+    for src in SOURCES:
+        obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+        objs.append(obj)
+        cmd = [cc] + HIPCC_FLAGS + (["-x", "hip"] if src.endswith(".cpp") else []) + \
+              ["-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    for src, p in procs:
+        out, _ = p.communicate()
+        out = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l)
+        if p.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}:\n{out}")
+        if verbose and out.strip():
+            print(out, flush=True)
+    tmp = LIB_PATH + ".tmp"
+    link = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + objs
+    r = subprocess.run(link, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stdout}")
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(force="--force" in sys.argv or needs_build(), verbose=True))

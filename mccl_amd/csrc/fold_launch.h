@@ -1,0 +1,62 @@
+// fold_launch.h -- host/device shared argument blocks of the fold kernels and
+// the internal launch entry used by the C ABI (mcclx_api.cpp).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mcclx.h"
+
+namespace mcclx {
+
+constexpr int kFewSegs = 8;  // segments that travel by value in the kernel arguments
+
+// Device-side view of mcclx_seg (same layout: the table is uploaded verbatim).
+struct SegArgs {
+    void* out;
+    void* wire_out;
+    const void* in[MCCLX_MAX_INPUTS];
+    uint64_t count;
+};
+static_assert(sizeof(SegArgs) == sizeof(mcclx_seg), "SegArgs must mirror mcclx_seg");
+
+struct FewArgs {
+    SegArgs seg[kFewSegs];
+    float scale;        // the constant as the fp32 value the kernel multiplies by
+    int32_t has_scale;
+    int32_t nseg;
+};
+
+struct TableArgs {
+    const SegArgs* __restrict__ segs;         // device memory, nseg entries
+    const uint64_t* __restrict__ first_item;  // device memory, nseg+1 prefix sums (unused when uniform)
+    uint64_t total_items;
+    uint64_t uniform_items;      // >0: every segment has this many work items
+    uint32_t nseg;
+    float scale;
+    int32_t has_scale;
+};
+
+struct PlanKey {
+    int dtype, io, k, topo, op, acc;
+};
+
+struct LaunchParams {
+    const FewArgs* few = nullptr;      // exactly one of few / table is set
+    const TableArgs* table = nullptr;
+    uint32_t max_blocks = 0;           // cap on the grid (persistent sizing)
+};
+
+// Packets-per-lane unroll the kernel template uses for this plan.
+int plan_unroll(const PlanKey& key);
+// Work items (tiles) a segment of `count` elements splits into under this plan.
+uint32_t items_for(const PlanKey& key, uint64_t count);
+// hipErrorInvalidValue = no kernel for this plan.
+hipError_t launch_fold(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
+
+// Plain device copy with the same packet shape (also the calibration kernel for
+// the memory counters): dst <- src, nbytes.
+hipError_t launch_copy(hipStream_t st, void* dst, const void* src, uint64_t nbytes,
+                       uint32_t max_blocks);
+
+}  // namespace mcclx

@@ -1,0 +1,790 @@
+// mcclx_api.cpp -- the C ABI (include/mcclx.h): context, reduce queue, launch
+// validation, host-buffer interop.  Host-only code; kernels live in
+// fold_kernels.hip / copy_kernel.hip behind fold_launch.h.
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "fold_launch.h"
+#include "mcclx.h"
+#include "mcclx_internal.h"
+
+namespace {
+thread_local std::string g_err;
+}
+
+extern "C" int mcclx_fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    // same prefix as the reference's MCCLError (csrc/common/Errors.hpp:9-13)
+    g_err = std::string("[MCCL] ") + buf;
+    return code;
+}
+
+namespace {
+
+#define fail mcclx_fail
+
+#define HIP_TRY(expr)                                                                  \
+    do {                                                                               \
+        hipError_t _e = (expr);                                                        \
+        if (_e != hipSuccess)                                                          \
+            return fail(MCCLX_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(_e)); \
+    } while (0)
+
+constexpr int kTableSlots = 4;
+
+struct TableSlot {
+    void* host = nullptr;  // pinned staging
+    void* dev = nullptr;
+    size_t cap = 0;
+    hipEvent_t done = nullptr;  // recorded after the launch that read `dev`
+    bool pending = false;
+};
+
+}  // namespace
+
+struct mcclx_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    std::vector<void*> tables;  // descriptor tables recorded launches read
+};
+
+struct mcclx_ctx {
+    bool capturing = false;
+    std::vector<void*> capture_tables;
+    int device = 0;
+    hipStream_t stream = nullptr;
+    bool own_stream = false;
+    int cus = 0;
+    uint32_t max_blocks = 0;
+    bool validate = false;
+    bool batch_active = false;
+    std::string batch_label;
+    std::mutex mu;
+    std::unordered_map<uint64_t, hipEvent_t> tickets;
+    std::vector<hipEvent_t> free_events;
+    uint64_t next_ticket = 1;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    bool timing = false;
+    TableSlot slots[kTableSlots];
+    int next_slot = 0;
+    std::unordered_map<void*, uint64_t> host_allocs;
+    // cross-stream ordering events, used round robin so that an event is not
+    // re-recorded until 15 later waits have been issued
+    hipEvent_t xev[16] = {};
+    int xnext = 0;
+};
+
+namespace {
+
+bool dtype_ok(int d) { return d == MCCLX_F32 || d == MCCLX_F16 || d == MCCLX_BF16; }
+
+struct DeviceGuard {
+    int prev = -1;
+    bool ok = true;
+    explicit DeviceGuard(int dev) {
+        if (hipGetDevice(&prev) != hipSuccess) prev = -1;
+        if (prev != dev) ok = (hipSetDevice(dev) == hipSuccess);
+    }
+    ~DeviceGuard() {
+        if (prev >= 0) (void)hipSetDevice(prev);
+    }
+};
+
+// binary16 <- binary64 in one rounding (the `(__fp16)scale` of
+// MetalKernels.mm:387,656): scale into the target's quantum, round to nearest
+// even with nearbyint (exact in double), rebuild the pattern.
+uint16_t f64_to_f16_bits(double x) {
+    uint16_t sign = std::signbit(x) ? 0x8000u : 0u;
+    double a = std::fabs(x);
+    if (std::isnan(x)) return (uint16_t)(sign | 0x7E00u);
+    if (std::isinf(x)) return (uint16_t)(sign | 0x7C00u);
+    if (a == 0.0) return sign;
+    int e;
+    double m = std::frexp(a, &e);  // a = m * 2^e, m in [0.5, 1)
+    if (e < -13) {                 // below the smallest normal 2^-14: fixed quantum 2^-24
+        double q = std::nearbyint(std::ldexp(a, 24));
+        return (uint16_t)(sign | (uint16_t)q);  // q == 1024 is the smallest normal
+    }
+    double q = std::nearbyint(std::ldexp(m, 11));  // 11 significant bits: [1024, 2048]
+    if (q == 2048.0) {
+        q = 1024.0;
+        e += 1;
+    }
+    int field = e + 14;
+    if (field >= 31) return (uint16_t)(sign | 0x7C00u);
+    return (uint16_t)(sign | (field << 10) | ((int)q - 1024));
+}
+
+float f16_bits_to_f32(uint16_t h) {
+    int ex = (h >> 10) & 0x1F, man = h & 0x3FF;
+    double v;
+    if (ex == 0)
+        v = std::ldexp((double)man, -24);
+    else if (ex == 31)
+        v = man ? NAN : INFINITY;
+    else
+        v = std::ldexp((double)(man | 0x400), ex - 25);
+    return (float)((h & 0x8000) ? -v : v);
+}
+
+// The multiplier each scale kernel receives, as an fp32 value
+// (MetalKernels.mm:384-398 tensor variant, :655-666 view variant).
+int scale_value(int dtype, double scale, int mode, float* out) {
+    float f = (float)scale;
+    uint32_t bits;
+    memcpy(&bits, &f, 4);
+    if (dtype == MCCLX_F32) {
+        *out = f;
+    } else if (dtype == MCCLX_F16) {
+        *out = f16_bits_to_f32(f64_to_f16_bits(scale));
+    } else if (mode == MCCLX_SCALE_VIEW) {
+        bits &= 0xFFFF0000u;  // bits >> 16, truncation
+        memcpy(out, &bits, 4);
+    } else if (mode == MCCLX_SCALE_TENSOR) {
+        if ((bits & 0x7FFFFFFFu) > 0x7F800000u)
+            bits = 0x7FC00000u;
+        else
+            bits = (bits + 0x7FFFu + ((bits >> 16) & 1u)) & 0xFFFF0000u;
+        memcpy(out, &bits, 4);
+    } else {
+        return fail(MCCLX_ERR_INVALID, "scale_mode %d is not VIEW or TENSOR", mode);
+    }
+    return MCCLX_OK;
+}
+
+int normalize_op(int op, int* out) {
+    switch (op) {
+        case MCCLX_SUM:
+        case MCCLX_AVG: *out = MCCLX_SUM; return MCCLX_OK;  // select_op_pipeline, MetalKernels.mm:609-611
+        case MCCLX_PRODUCT:
+        case MCCLX_MIN:
+        case MCCLX_MAX: *out = op; return MCCLX_OK;
+        default:
+            // MetalKernels.mm:546-548
+            return fail(MCCLX_ERR_UNSUPPORTED, "Unsupported ReduceOp: %d", op);
+    }
+}
+
+int check_plan(const mcclx_plan* p, mcclx::PlanKey* key, float* scale_f, int* has_scale) {
+    if (!p) return fail(MCCLX_ERR_INVALID, "plan is null");
+    if (p->reserved != 0) return fail(MCCLX_ERR_INVALID, "plan.reserved must be 0");
+    if (!dtype_ok(p->dtype))
+        return fail(MCCLX_ERR_UNSUPPORTED, "No kernel for dtype code %d", p->dtype);
+    if (p->k < 1 || p->k > MCCLX_MAX_INPUTS)
+        return fail(MCCLX_ERR_INVALID, "plan.k=%d outside 1..%d", p->k, MCCLX_MAX_INPUTS);
+    int op;
+    if (int rc = normalize_op(p->op, &op)) return rc;
+    if (p->io < MCCLX_IO_PURE || p->io > MCCLX_IO_OWN_LAST_F32)
+        return fail(MCCLX_ERR_INVALID, "plan.io=%d unknown", p->io);
+    if (p->io != MCCLX_IO_PURE && p->dtype != MCCLX_BF16)
+        return fail(MCCLX_ERR_UNSUPPORTED, "fp32 operands/outputs need the bf16 wire dtype");
+    if (p->topo != MCCLX_TOPO_FOLD && p->topo != MCCLX_TOPO_BINOMIAL)
+        return fail(MCCLX_ERR_INVALID, "plan.topo=%d unknown", p->topo);
+    if (p->acc != MCCLX_ACC_STEP && p->acc != MCCLX_ACC_F32)
+        return fail(MCCLX_ERR_INVALID, "plan.acc=%d unknown", p->acc);
+    if (op != MCCLX_SUM && (p->k > 2 || p->io != MCCLX_IO_PURE || p->acc != MCCLX_ACC_STEP))
+        return fail(MCCLX_ERR_UNSUPPORTED,
+                    "MIN/MAX/PRODUCT run as the reference's binary kernels only (k<=2, PURE, STEP)");
+    if (p->dtype == MCCLX_F16 && (p->k > 2 || p->acc != MCCLX_ACC_STEP))
+        return fail(MCCLX_ERR_UNSUPPORTED, "fp16 runs as the reference's binary kernels only (k<=2)");
+    if (p->io == MCCLX_IO_OWN_LAST_F32 && p->topo == MCCLX_TOPO_BINOMIAL)
+        return fail(MCCLX_ERR_UNSUPPORTED, "the tree reduces into rank 0: own operand is first");
+    int acc = (p->dtype == MCCLX_F32) ? MCCLX_ACC_STEP : p->acc;  // fp32 has no rounding to skip
+    *key = mcclx::PlanKey{p->dtype, p->io, p->k, (p->k >= 4) ? p->topo : MCCLX_TOPO_FOLD, op, acc};
+    *has_scale = p->scale_mode != MCCLX_SCALE_NONE;
+    *scale_f = 1.0f;
+    if (*has_scale)
+        if (int rc = scale_value(p->dtype, p->scale, p->scale_mode, scale_f)) return rc;
+    return MCCLX_OK;
+}
+
+bool in_is_f32(const mcclx::PlanKey& k, int i) {
+    return k.dtype == MCCLX_F32 || (k.io == MCCLX_IO_OWN_FIRST_F32 && i == 0) ||
+           (k.io == MCCLX_IO_OWN_LAST_F32 && i == k.k - 1);
+}
+
+// Is [p, p+nbytes) inside one allocation the GPU can address?
+int check_range(const void* p, uint64_t nbytes, const char* what, uint32_t seg) {
+    hipPointerAttribute_t attr;
+    hipError_t e = hipPointerGetAttributes(&attr, p);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(MCCLX_ERR_INVALID, "segment %u: %s=%p is not GPU-accessible memory", seg, what, p);
+    }
+    void* base = nullptr;
+    size_t size = 0;
+    if (attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged) {
+        if (hipMemGetAddressRange((hipDeviceptr_t*)&base, &size, (hipDeviceptr_t)p) != hipSuccess) {
+            (void)hipGetLastError();
+            return MCCLX_OK;  // range unknown: accept
+        }
+        const char* lo = static_cast<const char*>(base);
+        const char* q = static_cast<const char*>(p);
+        if (q < lo || q + nbytes > lo + size)
+            return fail(MCCLX_ERR_INVALID,
+                        "segment %u: %s=%p + %llu bytes runs past its allocation (%zu bytes at %p)",
+                        seg, what, p, (unsigned long long)nbytes, size, base);
+    }
+    return MCCLX_OK;
+}
+
+int check_segs(mcclx_ctx* ctx, const mcclx::PlanKey& key, const mcclx_seg* segs, uint32_t nseg) {
+    if (!segs && nseg) return fail(MCCLX_ERR_INVALID, "segment array is null");
+    const bool out_f32 = key.dtype == MCCLX_F32 || key.io != MCCLX_IO_PURE;
+    for (uint32_t s = 0; s < nseg; ++s) {
+        const mcclx_seg& g = segs[s];
+        if (g.count == 0) continue;
+        if (!g.out && !g.wire_out) return fail(MCCLX_ERR_INVALID, "segment %u has no output", s);
+        if (g.wire_out && key.dtype == MCCLX_F32)
+            return fail(MCCLX_ERR_INVALID, "segment %u: wire_out needs a 16-bit arithmetic dtype", s);
+        for (int i = 0; i < key.k; ++i) {
+            if (!g.in[i]) return fail(MCCLX_ERR_INVALID, "segment %u: in[%d] is null", s, i);
+            size_t al = in_is_f32(key, i) ? 4 : 2;
+            if ((uintptr_t)g.in[i] % al)
+                return fail(MCCLX_ERR_INVALID, "segment %u: in[%d]=%p is not element aligned", s, i,
+                            g.in[i]);
+        }
+        if (g.out && (uintptr_t)g.out % (out_f32 ? 4 : 2))
+            return fail(MCCLX_ERR_INVALID, "segment %u: out=%p is not element aligned", s, g.out);
+        if (g.wire_out && (uintptr_t)g.wire_out % 2)
+            return fail(MCCLX_ERR_INVALID, "segment %u: wire_out=%p is not element aligned", s,
+                        g.wire_out);
+        if (ctx->validate) {
+            for (int i = 0; i < key.k; ++i)
+                if (int rc = check_range(g.in[i], g.count * (in_is_f32(key, i) ? 4 : 2), "in", s))
+                    return rc;
+            if (g.out)
+                if (int rc = check_range(g.out, g.count * (out_f32 ? 4 : 2), "out", s)) return rc;
+            if (g.wire_out)
+                if (int rc = check_range(g.wire_out, g.count * 2, "wire_out", s)) return rc;
+        }
+    }
+    return MCCLX_OK;
+}
+
+int launch_error(hipError_t e, const mcclx::PlanKey& k) {
+    if (e == hipErrorInvalidValue)
+        return fail(MCCLX_ERR_UNSUPPORTED, "No kernel for plan dtype=%d io=%d k=%d topo=%d op=%d acc=%d",
+                    k.dtype, k.io, k.k, k.topo, k.op, k.acc);
+    return fail(MCCLX_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+}
+
+int ensure_slot(mcclx_ctx* ctx, TableSlot& sl, size_t need) {
+    if (sl.pending) {
+        HIP_TRY(hipEventSynchronize(sl.done));
+        sl.pending = false;
+    }
+    if (sl.cap >= need) return MCCLX_OK;
+    size_t cap = 1 << 16;
+    while (cap < need) cap <<= 1;
+    if (sl.host) HIP_TRY(hipHostFree(sl.host));
+    if (sl.dev) HIP_TRY(hipFree(sl.dev));
+    sl.host = sl.dev = nullptr;
+    sl.cap = 0;
+    HIP_TRY(hipHostMalloc(&sl.host, cap, hipHostMallocDefault));
+    HIP_TRY(hipMalloc(&sl.dev, cap));
+    if (!sl.done) HIP_TRY(hipEventCreateWithFlags(&sl.done, hipEventDisableTiming));
+    sl.cap = cap;
+    (void)ctx;
+    return MCCLX_OK;
+}
+
+int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uint32_t nseg) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    mcclx::PlanKey key;
+    float scale_f;
+    int has_scale;
+    if (int rc = check_plan(plan, &key, &scale_f, &has_scale)) return rc;
+    if (int rc = check_segs(ctx, key, segs, nseg)) return rc;
+    if (nseg == 0) return MCCLX_OK;
+    DeviceGuard guard(ctx->device);
+    if (!guard.ok) return fail(MCCLX_ERR_HIP, "hipSetDevice(%d) failed", ctx->device);
+
+    mcclx::LaunchParams lp;
+    lp.max_blocks = ctx->max_blocks;
+    if (nseg <= (uint32_t)mcclx::kFewSegs) {
+        mcclx::FewArgs a;
+        memset(&a, 0, sizeof a);
+        for (uint32_t s = 0; s < nseg; ++s) memcpy(&a.seg[s], &segs[s], sizeof(mcclx_seg));
+        a.scale = scale_f;
+        a.has_scale = has_scale;
+        a.nseg = (int32_t)nseg;
+        lp.few = &a;
+        hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
+        if (e != hipSuccess) return launch_error(e, key);
+        return MCCLX_OK;
+    }
+
+    // descriptor table: segs, then nseg+1 work-item prefix sums
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    size_t seg_bytes = (size_t)nseg * sizeof(mcclx_seg);
+    size_t pre_bytes = ((size_t)nseg + 1) * sizeof(uint64_t);
+    if (ctx->capturing) {
+        // A recorded launch needs a table that outlives this call: give it its
+        // own device buffer, filled now with a blocking copy (outside the
+        // recording), owned by the graph.
+        std::vector<char> host(seg_bytes + pre_bytes);
+        memcpy(host.data(), segs, seg_bytes);
+        uint64_t* pre = reinterpret_cast<uint64_t*>(host.data() + seg_bytes);
+        uint64_t total = 0, uniform = mcclx::items_for(key, segs[0].count);
+        for (uint32_t s = 0; s < nseg; ++s) {
+            pre[s] = total;
+            uint64_t n = mcclx::items_for(key, segs[s].count);
+            if (n != uniform) uniform = 0;
+            total += n;
+        }
+        pre[nseg] = total;
+        if (total == 0) return MCCLX_OK;
+        void* dev = nullptr;
+        HIP_TRY(hipMalloc(&dev, host.size()));
+        hipError_t ce = hipMemcpy(dev, host.data(), host.size(), hipMemcpyHostToDevice);
+        if (ce != hipSuccess) {
+            (void)hipFree(dev);
+            return fail(MCCLX_ERR_HIP, "table upload failed: %s", hipGetErrorString(ce));
+        }
+        ctx->capture_tables.push_back(dev);
+        mcclx::TableArgs t;
+        t.segs = static_cast<const mcclx::SegArgs*>(dev);
+        t.first_item = reinterpret_cast<const uint64_t*>(static_cast<char*>(dev) + seg_bytes);
+        t.total_items = total;
+        t.uniform_items = uniform;
+        t.nseg = nseg;
+        t.scale = scale_f;
+        t.has_scale = has_scale;
+        lp.table = &t;
+        hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
+        if (e != hipSuccess) return launch_error(e, key);
+        return MCCLX_OK;
+    }
+    TableSlot& sl = ctx->slots[ctx->next_slot];
+    ctx->next_slot = (ctx->next_slot + 1) % kTableSlots;
+    if (int rc = ensure_slot(ctx, sl, seg_bytes + pre_bytes)) return rc;
+    memcpy(sl.host, segs, seg_bytes);
+    uint64_t* pre = reinterpret_cast<uint64_t*>(static_cast<char*>(sl.host) + seg_bytes);
+    uint64_t total = 0, uniform = mcclx::items_for(key, segs[0].count);
+    for (uint32_t s = 0; s < nseg; ++s) {
+        pre[s] = total;
+        uint64_t n = mcclx::items_for(key, segs[s].count);
+        if (n != uniform) uniform = 0;
+        total += n;
+    }
+    pre[nseg] = total;
+    if (total == 0) return MCCLX_OK;
+    HIP_TRY(hipMemcpyAsync(sl.dev, sl.host, seg_bytes + pre_bytes, hipMemcpyHostToDevice, ctx->stream));
+    mcclx::TableArgs t;
+    t.segs = static_cast<const mcclx::SegArgs*>(sl.dev);
+    t.first_item = reinterpret_cast<const uint64_t*>(static_cast<char*>(sl.dev) + seg_bytes);
+    t.total_items = total;
+    t.uniform_items = uniform;
+    t.nseg = nseg;
+    t.scale = scale_f;
+    t.has_scale = has_scale;
+    lp.table = &t;
+    hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
+    if (e != hipSuccess) return launch_error(e, key);
+    HIP_TRY(hipEventRecord(sl.done, ctx->stream));
+    sl.pending = true;
+    return MCCLX_OK;
+}
+
+int make_ctx(int device, hipStream_t borrowed, bool borrow, mcclx_ctx** out) {
+    if (!out) return fail(MCCLX_ERR_INVALID, "out is null");
+    *out = nullptr;
+    int n = 0;
+    HIP_TRY(hipGetDeviceCount(&n));
+    if (device < 0 || device >= n)
+        return fail(MCCLX_ERR_INVALID, "device %d out of range (%d visible)", device, n);
+    DeviceGuard guard(device);
+    if (!guard.ok) return fail(MCCLX_ERR_HIP, "hipSetDevice(%d) failed", device);
+    auto* ctx = new mcclx_ctx();
+    ctx->device = device;
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) {
+        delete ctx;
+        return fail(MCCLX_ERR_HIP, "hipGetDeviceProperties failed: %s", hipGetErrorString(e));
+    }
+    ctx->cus = prop.multiProcessorCount;
+    int per_cu = 32;
+    if (const char* v = getenv("MCCLX_BLOCKS_PER_CU")) {
+        int x = atoi(v);
+        if (x >= 1 && x <= 1024) per_cu = x;
+    }
+    ctx->max_blocks = (uint32_t)ctx->cus * (uint32_t)per_cu;
+    if (const char* v = getenv("MCCLX_VALIDATE")) ctx->validate = (v[0] == '1');
+    if (borrow) {
+        ctx->stream = borrowed;
+    } else {
+        e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);  // default priority
+        if (e != hipSuccess) {
+            delete ctx;
+            return fail(MCCLX_ERR_HIP, "hipStreamCreateWithFlags failed: %s", hipGetErrorString(e));
+        }
+        ctx->own_stream = true;
+    }
+    *out = ctx;
+    return MCCLX_OK;
+}
+
+int get_event(mcclx_ctx* ctx, hipEvent_t* ev) {
+    if (!ctx->free_events.empty()) {
+        *ev = ctx->free_events.back();
+        ctx->free_events.pop_back();
+        return MCCLX_OK;
+    }
+    HIP_TRY(hipEventCreateWithFlags(ev, hipEventDisableTiming));
+    return MCCLX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* mcclx_last_error(void) { return g_err.c_str(); }
+int mcclx_abi_version(void) { return MCCLX_ABI_VERSION; }
+
+int mcclx_init(int device, mcclx_ctx** out) { return make_ctx(device, nullptr, false, out); }
+
+int mcclx_init_on_stream(int device, void* hip_stream, mcclx_ctx** out) {
+    return make_ctx(device, static_cast<hipStream_t>(hip_stream), true, out);
+}
+
+int mcclx_destroy(mcclx_ctx* ctx) {
+    if (!ctx) return MCCLX_OK;
+    DeviceGuard guard(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    for (auto& kv : ctx->tickets) (void)hipEventDestroy(kv.second);
+    for (auto ev : ctx->free_events) (void)hipEventDestroy(ev);
+    for (auto ev : ctx->xev)
+        if (ev) (void)hipEventDestroy(ev);
+    if (ctx->t0) (void)hipEventDestroy(ctx->t0);
+    if (ctx->t1) (void)hipEventDestroy(ctx->t1);
+    for (auto& sl : ctx->slots) {
+        if (sl.host) (void)hipHostFree(sl.host);
+        if (sl.dev) (void)hipFree(sl.dev);
+        if (sl.done) (void)hipEventDestroy(sl.done);
+    }
+    for (auto& kv : ctx->host_allocs) (void)hipHostFree(kv.first);
+    if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return MCCLX_OK;
+}
+
+void* mcclx_queue_stream(mcclx_ctx* ctx) { return ctx ? (void*)ctx->stream : nullptr; }
+int mcclx_device_cus(mcclx_ctx* ctx) { return ctx ? ctx->cus : 0; }
+
+int mcclx_fold(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* seg) {
+    return fold_impl(ctx, plan, seg, 1);
+}
+
+int mcclx_fold_batched(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uint32_t nseg) {
+    return fold_impl(ctx, plan, segs, nseg);
+}
+
+int mcclx_reduce(mcclx_ctx* ctx, void* dst, const void* src, int dtype, uint64_t count, int op) {
+    mcclx_plan p = {dtype, MCCLX_IO_PURE, 2, MCCLX_TOPO_FOLD, op, MCCLX_ACC_STEP, MCCLX_SCALE_NONE, 0, 0.0};
+    mcclx_seg s;
+    memset(&s, 0, sizeof s);
+    s.out = dst;
+    s.in[0] = dst;
+    s.in[1] = src;
+    s.count = count;
+    return fold_impl(ctx, &p, &s, 1);
+}
+
+int mcclx_scale(mcclx_ctx* ctx, void* buf, int dtype, uint64_t count, double scale, int scale_mode) {
+    if (scale_mode != MCCLX_SCALE_VIEW && scale_mode != MCCLX_SCALE_TENSOR)
+        return fail(MCCLX_ERR_INVALID, "scale_mode %d is not VIEW or TENSOR", scale_mode);
+    mcclx_plan p = {dtype, MCCLX_IO_PURE, 1, MCCLX_TOPO_FOLD, MCCLX_SUM, MCCLX_ACC_STEP, scale_mode, 0, scale};
+    mcclx_seg s;
+    memset(&s, 0, sizeof s);
+    s.out = buf;
+    s.in[0] = buf;
+    s.count = count;
+    return fold_impl(ctx, &p, &s, 1);
+}
+
+int mcclx_accumulate_scale(mcclx_ctx* ctx, void* dst, const void* src, int dtype, uint64_t count,
+                           double scale) {
+    mcclx_plan p = {dtype, MCCLX_IO_PURE, 2, MCCLX_TOPO_FOLD, MCCLX_SUM, MCCLX_ACC_STEP,
+                    MCCLX_SCALE_TENSOR, 0, scale};
+    mcclx_seg s;
+    memset(&s, 0, sizeof s);
+    s.out = dst;
+    s.in[0] = dst;
+    s.in[1] = src;
+    s.count = count;
+    return fold_impl(ctx, &p, &s, 1);
+}
+
+int mcclx_encode_bf16(mcclx_ctx* ctx, void* dst_bf16, const void* src_f32, uint64_t count) {
+    mcclx_plan p = {MCCLX_BF16, MCCLX_IO_OWN_FIRST_F32, 1, MCCLX_TOPO_FOLD, MCCLX_SUM, MCCLX_ACC_STEP,
+                    MCCLX_SCALE_NONE, 0, 0.0};
+    mcclx_seg s;
+    memset(&s, 0, sizeof s);
+    s.wire_out = dst_bf16;
+    s.in[0] = src_f32;
+    s.count = count;
+    return fold_impl(ctx, &p, &s, 1);
+}
+
+int mcclx_decode_bf16(mcclx_ctx* ctx, void* dst_f32, const void* src_bf16, uint64_t count) {
+    mcclx_plan p = {MCCLX_BF16, MCCLX_IO_OUT_F32, 1, MCCLX_TOPO_FOLD, MCCLX_SUM, MCCLX_ACC_STEP,
+                    MCCLX_SCALE_NONE, 0, 0.0};
+    mcclx_seg s;
+    memset(&s, 0, sizeof s);
+    s.out = dst_f32;
+    s.in[0] = src_bf16;
+    s.count = count;
+    return fold_impl(ctx, &p, &s, 1);
+}
+
+int mcclx_copy(mcclx_ctx* ctx, void* dst, const void* src, uint64_t nbytes) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    if (nbytes == 0 || dst == src) return MCCLX_OK;
+    if (!dst || !src) return fail(MCCLX_ERR_INVALID, "copy: null pointer");
+    if (ctx->validate) {
+        if (int rc = check_range(src, nbytes, "src", 0)) return rc;
+        if (int rc = check_range(dst, nbytes, "dst", 0)) return rc;
+    }
+    DeviceGuard guard(ctx->device);
+    hipError_t e = mcclx::launch_copy(ctx->stream, dst, src, nbytes, ctx->max_blocks);
+    if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "copy launch failed: %s", hipGetErrorString(e));
+    return MCCLX_OK;
+}
+
+int mcclx_batch_begin(mcclx_ctx* ctx, const char* label) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    if (ctx->batch_active) return fail(MCCLX_ERR_STATE, "batch already active");  // MetalKernels.mm:562
+    ctx->batch_active = true;
+    ctx->batch_label = label ? label : "mccl_batch";
+    return MCCLX_OK;
+}
+
+int mcclx_batch_end(mcclx_ctx* ctx) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    ctx->batch_active = false;  // no-op when none is open (MetalKernels.mm:571)
+    return MCCLX_OK;
+}
+
+#define REFUSE_WHILE_RECORDING(ctx, what)                                                     \
+    if ((ctx)->capturing)                                                                    \
+    return fail(MCCLX_ERR_STATE, what " is not allowed between graph_begin and graph_end")
+
+int mcclx_queue_drain(mcclx_ctx* ctx) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    REFUSE_WHILE_RECORDING(ctx, "queue_drain");
+    DeviceGuard guard(ctx->device);
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return MCCLX_OK;
+}
+
+static int stream_wait(mcclx_ctx* ctx, hipStream_t waiter, hipStream_t producer) {
+    if (waiter == producer) return MCCLX_OK;
+    REFUSE_WHILE_RECORDING(ctx, "cross-stream ordering");
+    DeviceGuard guard(ctx->device);
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    hipEvent_t& ev = ctx->xev[ctx->xnext];
+    ctx->xnext = (ctx->xnext + 1) % 16;
+    if (!ev) HIP_TRY(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    HIP_TRY(hipEventRecord(ev, producer));
+    HIP_TRY(hipStreamWaitEvent(waiter, ev, 0));
+    return MCCLX_OK;
+}
+
+int mcclx_queue_wait_stream(mcclx_ctx* ctx, void* producer_stream) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    return stream_wait(ctx, ctx->stream, static_cast<hipStream_t>(producer_stream));
+}
+
+int mcclx_stream_wait_queue(mcclx_ctx* ctx, void* consumer_stream) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    return stream_wait(ctx, static_cast<hipStream_t>(consumer_stream), ctx->stream);
+}
+
+int mcclx_event_record(mcclx_ctx* ctx, uint64_t* ticket) {
+    if (!ctx || !ticket) return fail(MCCLX_ERR_INVALID, "event_record: null argument");
+    REFUSE_WHILE_RECORDING(ctx, "event_record");
+    DeviceGuard guard(ctx->device);
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    hipEvent_t ev;
+    if (int rc = get_event(ctx, &ev)) return rc;
+    HIP_TRY(hipEventRecord(ev, ctx->stream));
+    *ticket = ctx->next_ticket++;
+    ctx->tickets[*ticket] = ev;
+    return MCCLX_OK;
+}
+
+int mcclx_event_query(mcclx_ctx* ctx, uint64_t ticket, int* done) {
+    if (!ctx || !done) return fail(MCCLX_ERR_INVALID, "event_query: null argument");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    auto it = ctx->tickets.find(ticket);
+    if (it == ctx->tickets.end()) {
+        // already waited for (or never issued): tickets below the counter are complete
+        if (ticket == 0 || ticket >= ctx->next_ticket) return fail(MCCLX_ERR_INVALID, "unknown ticket");
+        *done = 1;
+        return MCCLX_OK;
+    }
+    hipError_t e = hipEventQuery(it->second);
+    if (e == hipSuccess) {
+        *done = 1;
+    } else if (e == hipErrorNotReady) {
+        (void)hipGetLastError();
+        *done = 0;
+    } else {
+        return fail(MCCLX_ERR_HIP, "hipEventQuery failed: %s", hipGetErrorString(e));
+    }
+    return MCCLX_OK;
+}
+
+int mcclx_event_wait(mcclx_ctx* ctx, uint64_t ticket) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    if (ticket == 0) return MCCLX_OK;  // "fell back to blocking sync", MPSInterop.mm:352-355
+    hipEvent_t ev;
+    {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        auto it = ctx->tickets.find(ticket);
+        if (it == ctx->tickets.end()) {
+            if (ticket >= ctx->next_ticket) return fail(MCCLX_ERR_INVALID, "unknown ticket");
+            return MCCLX_OK;
+        }
+        ev = it->second;
+        ctx->tickets.erase(it);
+    }
+    hipError_t e = hipEventSynchronize(ev);
+    {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        ctx->free_events.push_back(ev);
+    }
+    if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "hipEventSynchronize failed: %s", hipGetErrorString(e));
+    return MCCLX_OK;
+}
+
+int mcclx_timer_begin(mcclx_ctx* ctx) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    REFUSE_WHILE_RECORDING(ctx, "timer_begin");
+    DeviceGuard guard(ctx->device);
+    if (!ctx->t0) {
+        HIP_TRY(hipEventCreate(&ctx->t0));
+        HIP_TRY(hipEventCreate(&ctx->t1));
+    }
+    HIP_TRY(hipEventRecord(ctx->t0, ctx->stream));
+    ctx->timing = true;
+    return MCCLX_OK;
+}
+
+int mcclx_timer_end(mcclx_ctx* ctx, float* elapsed_ms) {
+    if (!ctx || !elapsed_ms) return fail(MCCLX_ERR_INVALID, "timer_end: null argument");
+    if (!ctx->timing) return fail(MCCLX_ERR_STATE, "timer_end without timer_begin");
+    DeviceGuard guard(ctx->device);
+    HIP_TRY(hipEventRecord(ctx->t1, ctx->stream));
+    HIP_TRY(hipEventSynchronize(ctx->t1));
+    HIP_TRY(hipEventElapsedTime(elapsed_ms, ctx->t0, ctx->t1));
+    ctx->timing = false;
+    return MCCLX_OK;
+}
+
+int mcclx_graph_begin(mcclx_ctx* ctx) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    if (ctx->capturing) return fail(MCCLX_ERR_STATE, "graph recording already active");
+    DeviceGuard guard(ctx->device);
+    // relaxed mode: the blocking table uploads above stay legal while recording
+    HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+    ctx->capturing = true;
+    return MCCLX_OK;
+}
+
+int mcclx_graph_end(mcclx_ctx* ctx, mcclx_graph** out) {
+    if (!ctx || !out) return fail(MCCLX_ERR_INVALID, "graph_end: null argument");
+    if (!ctx->capturing) return fail(MCCLX_ERR_STATE, "graph_end without graph_begin");
+    DeviceGuard guard(ctx->device);
+    ctx->capturing = false;
+    auto* g = new mcclx_graph();
+    g->tables.swap(ctx->capture_tables);
+    hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
+    if (e == hipSuccess) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        if (g->graph) (void)hipGraphDestroy(g->graph);
+        for (void* t : g->tables) (void)hipFree(t);
+        delete g;
+        return fail(MCCLX_ERR_HIP, "graph_end failed: %s", hipGetErrorString(e));
+    }
+    *out = g;
+    return MCCLX_OK;
+}
+
+int mcclx_graph_launch(mcclx_ctx* ctx, mcclx_graph* graph) {
+    if (!ctx || !graph) return fail(MCCLX_ERR_INVALID, "graph_launch: null argument");
+    REFUSE_WHILE_RECORDING(ctx, "graph_launch");
+    DeviceGuard guard(ctx->device);
+    HIP_TRY(hipGraphLaunch(graph->exec, ctx->stream));
+    return MCCLX_OK;
+}
+
+int mcclx_graph_destroy(mcclx_ctx* ctx, mcclx_graph* graph) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    if (!graph) return MCCLX_OK;
+    DeviceGuard guard(ctx->device);
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+    if (graph->graph) (void)hipGraphDestroy(graph->graph);
+    for (void* t : graph->tables) (void)hipFree(t);
+    delete graph;
+    return MCCLX_OK;
+}
+
+int mcclx_host_alloc(mcclx_ctx* ctx, uint64_t nbytes, void** host_ptr, void** device_ptr) {
+    if (!ctx || !host_ptr || !device_ptr) return fail(MCCLX_ERR_INVALID, "host_alloc: null argument");
+    if (nbytes == 0) return fail(MCCLX_ERR_INVALID, "host_alloc: zero bytes");
+    DeviceGuard guard(ctx->device);
+    void* h = nullptr;
+    hipError_t e = hipHostMalloc(&h, nbytes, hipHostMallocMapped | hipHostMallocPortable);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(MCCLX_ERR_NOMEM, "hipHostMalloc(%llu) failed: %s", (unsigned long long)nbytes,
+                    hipGetErrorString(e));
+    }
+    void* d = nullptr;
+    e = hipHostGetDevicePointer(&d, h, 0);
+    if (e != hipSuccess) {
+        (void)hipHostFree(h);
+        return fail(MCCLX_ERR_HIP, "hipHostGetDevicePointer failed: %s", hipGetErrorString(e));
+    }
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    ctx->host_allocs[h] = nbytes;
+    *host_ptr = h;
+    *device_ptr = d;
+    return MCCLX_OK;
+}
+
+int mcclx_host_free(mcclx_ctx* ctx, void* host_ptr) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    if (!host_ptr) return MCCLX_OK;
+    {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        auto it = ctx->host_allocs.find(host_ptr);
+        if (it == ctx->host_allocs.end())
+            return fail(MCCLX_ERR_INVALID, "host_free: %p was not returned by mcclx_host_alloc", host_ptr);
+        ctx->host_allocs.erase(it);
+    }
+    DeviceGuard guard(ctx->device);
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipHostFree(host_ptr));
+    return MCCLX_OK;
+}
+
+}  // extern "C"

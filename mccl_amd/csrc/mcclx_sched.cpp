@@ -1,0 +1,497 @@
+// mcclx_sched.cpp -- the chunk scheduler: chunkize, algorithm selection and the
+// single-process replay of the ring / tree / butterfly allreduce schedules
+// (csrc/backend/AllreduceAlgos.cpp) plus reduce_scatter / allgather
+// (csrc/backend/ProcessGroupMCCL.cpp) for N virtual ranks on one GPU.
+//
+// Host C++ on top of the public C ABI only (mcclx_reduce, mcclx_fold_batched,
+// mcclx_copy, ...): nothing here touches HIP directly.
+//
+// STEPWISE mode issues the reference's launches one for one -- every send/recv
+// pair becomes a device copy into the receiver's scratch, followed by the
+// binary in-place reduce the reference runs on that scratch.
+// FUSED mode is the MI355X shape of the same schedule: for every chunk its
+// final owner folds all N operands in ONE pass, reading the peers' chunks where
+// they already lie (the position xGMI peer reads or a zero-copy host buffer
+// would put them in), rounding after each operand exactly as the stepwise
+// kernels would, so both modes give bit-identical tensors.
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "mcclx.h"
+#include "mcclx_internal.h"
+
+namespace {
+
+constexpr uint64_t kAlign = 256;  // workspace sub-buffers start on 256 B
+
+uint64_t align_up(uint64_t x) { return (x + kAlign - 1) / kAlign * kAlign; }
+uint64_t esize(int dtype) { return dtype == MCCLX_F32 ? 4 : 2; }
+
+struct Chunks {
+    std::vector<mcclx_chunk> c;
+    Chunks(int64_t numel, uint64_t es, int world) : c((size_t)world) {
+        mcclx_chunkize(numel, es, world, c.data());
+    }
+    const mcclx_chunk& operator[](int i) const { return c[(size_t)i]; }
+};
+
+char* at(void* base, uint64_t off) { return static_cast<char*>(base) + off; }
+const char* at(const void* base, uint64_t off) { return static_cast<const char*>(base) + off; }
+
+#define TRY(x)                 \
+    do {                       \
+        int _rc = (x);         \
+        if (_rc != MCCLX_OK) return _rc; \
+    } while (0)
+
+// recv scratch per rank, ProcessGroupMCCL.cpp:152-162
+uint64_t scratch_elems(int algo, int world, uint64_t numel) {
+    uint64_t per = (numel + (uint64_t)world - 1) / (uint64_t)world;
+    if (algo == MCCLX_ALGO_RING) return per;
+    if (algo == MCCLX_ALGO_BUTTERFLY) return (uint64_t)(world - 1) * per;
+    return numel;
+}
+
+struct Layout {
+    bool wire;
+    int wdtype;
+    uint64_t wire_stride;     // bytes between ranks' bf16 copies
+    uint64_t scratch_off;     // start of the recv scratch area
+    uint64_t scratch_stride;  // bytes between ranks' recv scratch
+    uint64_t total;
+};
+
+Layout layout_of(const mcclx_replay* r) {
+    Layout L;
+    L.wire = r->wire_bf16 && r->dtype == MCCLX_F32;  // ProcessGroupMCCL.cpp:131
+    L.wdtype = L.wire ? MCCLX_BF16 : r->dtype;
+    L.wire_stride = L.wire ? align_up(r->numel * 2) : 0;
+    L.scratch_off = L.wire_stride * (uint64_t)r->world;
+    bool need_scratch = r->mode == MCCLX_REPLAY_STEPWISE || r->world > MCCLX_MAX_INPUTS;
+    L.scratch_stride =
+        need_scratch ? align_up(scratch_elems(r->algo, r->world, r->numel) * esize(L.wdtype)) : 0;
+    L.total = L.scratch_off + L.scratch_stride * (uint64_t)r->world;
+    return L;
+}
+
+int bad(const char* msg) { return mcclx_fail(MCCLX_ERR_INVALID, "%s", msg); }
+
+// ---------------------------------------------------------------- STEPWISE
+
+int ring_stepwise(mcclx_ctx* ctx, int N, std::vector<void*>& t, std::vector<void*>& recv, int dtype,
+                  uint64_t numel, int op) {
+    Chunks c((int64_t)numel, esize(dtype), N);
+    for (int k = 0; k < N - 1; ++k) {  // AllreduceAlgos.cpp:62-75
+        for (int r = 0; r < N; ++r) {  // the wire: prev's send lands in r's scratch
+            int prev = (r - 1 + N) % N;
+            int idx = (r - k - 1 + N) % N;  // == prev's send_idx
+            TRY(mcclx_copy(ctx, recv[r], at(t[prev], c[idx].byte_off), c[idx].byte_len));
+        }
+        for (int r = 0; r < N; ++r) {
+            int idx = (r - k - 1 + N) % N;
+            TRY(mcclx_reduce(ctx, at(t[r], c[idx].byte_off), recv[r], dtype,
+                             (uint64_t)c[idx].elem_count, op));
+        }
+    }
+    for (int k = 0; k < N - 1; ++k)  // :77-86
+        for (int r = 0; r < N; ++r) {
+            int prev = (r - 1 + N) % N;
+            int idx = (r - k + N) % N;
+            TRY(mcclx_copy(ctx, at(t[r], c[idx].byte_off), at(t[prev], c[idx].byte_off),
+                           c[idx].byte_len));
+        }
+    return MCCLX_OK;
+}
+
+int tree_stepwise(mcclx_ctx* ctx, int N, std::vector<void*>& t, std::vector<void*>& recv, int dtype,
+                  uint64_t numel, int op) {
+    uint64_t nbytes = numel * esize(dtype);
+    std::vector<char> active((size_t)N, 1);
+    for (int mask = 1; mask < N; mask <<= 1) {  // AllreduceAlgos.cpp:100-114
+        for (int r = 0; r < N; ++r)
+            if (active[r] && (r & mask)) {
+                TRY(mcclx_copy(ctx, recv[r - mask], t[r], nbytes));
+                active[r] = 0;
+            }
+        for (int r = 0; r < N; ++r)
+            if (active[r] && !(r & mask) && r + mask < N)
+                TRY(mcclx_reduce(ctx, t[r], recv[r], dtype, numel, op));
+    }
+    int top = 1;
+    while (top * 2 < N) top <<= 1;
+    for (int mask = top; mask >= 1; mask >>= 1) {  // :119-126
+        int two = mask << 1;
+        for (int r = 0; r < N; ++r)
+            if ((r % two) == 0 && r + mask < N) TRY(mcclx_copy(ctx, t[r + mask], t[r], nbytes));
+    }
+    return MCCLX_OK;
+}
+
+int butterfly_stepwise(mcclx_ctx* ctx, int N, std::vector<void*>& t, std::vector<void*>& recv,
+                       int dtype, uint64_t numel, int op) {
+    Chunks c((int64_t)numel, esize(dtype), N);
+    for (int r = 0; r < N; ++r) {  // AllreduceAlgos.cpp:151-169
+        int slot = 0;
+        for (int p = 0; p < N; ++p) {
+            if (p == r) continue;
+            TRY(mcclx_copy(ctx, at(recv[r], (uint64_t)slot * c[r].byte_len),
+                           at(t[p], c[r].byte_off), c[r].byte_len));
+            slot++;
+        }
+    }
+    for (int r = 0; r < N; ++r)  // :172-180
+        for (int slot = 0; slot < N - 1; ++slot)
+            TRY(mcclx_reduce(ctx, at(t[r], c[r].byte_off), at(recv[r], (uint64_t)slot * c[r].byte_len),
+                             dtype, (uint64_t)c[r].elem_count, op));
+    for (int r = 0; r < N; ++r)  // :185-200
+        for (int p = 0; p < N; ++p)
+            if (p != r)
+                TRY(mcclx_copy(ctx, at(t[p], c[r].byte_off), at(t[r], c[r].byte_off), c[r].byte_len));
+    return MCCLX_OK;
+}
+
+int replay_stepwise(mcclx_ctx* ctx, const mcclx_replay* r, const Layout& L) {
+    const int N = r->world;
+    std::vector<void*> work((size_t)N), recv((size_t)N);
+    for (int i = 0; i < N; ++i) {
+        recv[i] = at(r->workspace, L.scratch_off + (uint64_t)i * L.scratch_stride);
+        if (L.wire) {
+            work[i] = at(r->workspace, (uint64_t)i * L.wire_stride);
+            TRY(mcclx_encode_bf16(ctx, work[i], r->tensors[i], r->numel));  // PG.cpp:131-132
+        } else {
+            work[i] = r->tensors[i];
+        }
+    }
+    if (r->algo == MCCLX_ALGO_RING)
+        TRY(ring_stepwise(ctx, N, work, recv, L.wdtype, r->numel, r->op));
+    else if (r->algo == MCCLX_ALGO_BUTTERFLY)
+        TRY(butterfly_stepwise(ctx, N, work, recv, L.wdtype, r->numel, r->op));
+    else
+        TRY(tree_stepwise(ctx, N, work, recv, L.wdtype, r->numel, r->op));
+    if (r->op == MCCLX_AVG)  // AllreduceAlgos.cpp:88-91,128-131,202-205
+        for (int i = 0; i < N; ++i)
+            TRY(mcclx_scale(ctx, work[i], L.wdtype, r->numel, 1.0 / (double)N, MCCLX_SCALE_VIEW));
+    if (L.wire)
+        for (int i = 0; i < N; ++i)  // PG.cpp:179-183
+            TRY(mcclx_decode_bf16(ctx, r->tensors[i], work[i], r->numel));
+    return MCCLX_OK;
+}
+
+// ------------------------------------------------------------------- FUSED
+
+mcclx_plan base_plan(const mcclx_replay* r, const Layout& L, int k) {
+    mcclx_plan p;
+    memset(&p, 0, sizeof p);
+    p.dtype = L.wdtype;
+    p.io = MCCLX_IO_PURE;
+    p.k = k;
+    p.topo = MCCLX_TOPO_FOLD;
+    p.op = r->op;
+    p.acc = r->acc;
+    p.scale_mode = (r->op == MCCLX_AVG) ? MCCLX_SCALE_VIEW : MCCLX_SCALE_NONE;
+    p.scale = 1.0 / (double)r->world;
+    return p;
+}
+
+// MIN / MAX / PRODUCT and fp16 only exist as binary kernels; a k-input fold of
+// those is k-1 launches accumulating into the output (same order, same result).
+int fold_any(mcclx_ctx* ctx, mcclx_plan p, std::vector<mcclx_seg>& segs) {
+    bool binary_only = (p.op != MCCLX_SUM && p.op != MCCLX_AVG) || p.dtype == MCCLX_F16;
+    if (!binary_only || p.k <= 2) return mcclx_fold_batched(ctx, &p, segs.data(), (uint32_t)segs.size());
+    if (p.topo == MCCLX_TOPO_BINOMIAL) return MCCLX_ERR_UNSUPPORTED;  // caller uses STEPWISE
+    const int K = p.k;
+    int scale_mode = p.scale_mode;
+    for (int j = 1; j < K; ++j) {
+        mcclx_plan q = p;
+        q.k = 2;
+        q.scale_mode = (j == K - 1) ? scale_mode : MCCLX_SCALE_NONE;
+        std::vector<mcclx_seg> step(segs.size());
+        for (size_t s = 0; s < segs.size(); ++s) {
+            memset(&step[s], 0, sizeof(mcclx_seg));
+            step[s].out = segs[s].out;
+            step[s].in[0] = (j == 1) ? segs[s].in[0] : segs[s].out;
+            step[s].in[1] = segs[s].in[j];
+            step[s].count = segs[s].count;
+        }
+        TRY(mcclx_fold_batched(ctx, &q, step.data(), (uint32_t)step.size()));
+    }
+    return MCCLX_OK;
+}
+
+int replay_fused(mcclx_ctx* ctx, const mcclx_replay* r, const Layout& L) {
+    const int N = r->world;
+    const uint64_t es = esize(L.wdtype);  // element size on the "wire"
+    const uint64_t ts = esize(r->dtype);  // element size of the rank tensors
+    auto wire_of = [&](int rank) -> void* { return at(r->workspace, (uint64_t)rank * L.wire_stride); };
+    std::vector<mcclx_seg> segs;
+    mcclx_seg z;
+    memset(&z, 0, sizeof z);
+
+    if (r->algo == MCCLX_ALGO_TREE) {
+        // allreduce_tree: rank 0 ends with the binomial combination of all
+        // tensors (AllreduceAlgos.cpp:100-114), everyone else receives a copy.
+        mcclx_plan p = base_plan(r, L, N);
+        p.topo = MCCLX_TOPO_BINOMIAL;
+        if (L.wire) {
+            mcclx_plan e = base_plan(r, L, 1);  // encode ranks 1.. (their tensors travel)
+            e.io = MCCLX_IO_OWN_FIRST_F32;
+            e.op = MCCLX_SUM;
+            e.scale_mode = MCCLX_SCALE_NONE;
+            for (int q = 1; q < N; ++q) {
+                mcclx_seg s = z;
+                s.wire_out = wire_of(q);
+                s.in[0] = r->tensors[q];
+                s.count = r->numel;
+                segs.push_back(s);
+            }
+            if (!segs.empty()) TRY(mcclx_fold_batched(ctx, &e, segs.data(), (uint32_t)segs.size()));
+            segs.clear();
+            p.io = MCCLX_IO_OWN_FIRST_F32;
+        }
+        mcclx_seg s = z;
+        s.out = r->tensors[0];
+        s.count = r->numel;
+        s.in[0] = r->tensors[0];
+        for (int q = 1; q < N; ++q) s.in[q] = L.wire ? wire_of(q) : r->tensors[q];
+        if (L.wire) s.wire_out = wire_of(0);
+        segs.push_back(s);
+        TRY(fold_any(ctx, p, segs));
+        segs.clear();
+        if (L.wire) {  // broadcast of the bf16 result + the final cast on every rank
+            mcclx_plan d = base_plan(r, L, 1);
+            d.io = MCCLX_IO_OUT_F32;
+            d.op = MCCLX_SUM;
+            d.scale_mode = MCCLX_SCALE_NONE;
+            for (int q = 1; q < N; ++q) {
+                mcclx_seg g = z;
+                g.out = r->tensors[q];
+                g.in[0] = wire_of(0);
+                g.count = r->numel;
+                segs.push_back(g);
+            }
+            if (!segs.empty()) TRY(mcclx_fold_batched(ctx, &d, segs.data(), (uint32_t)segs.size()));
+        } else {
+            for (int q = 1; q < N; ++q) TRY(mcclx_copy(ctx, r->tensors[q], r->tensors[0], r->numel * ts));
+        }
+        return MCCLX_OK;
+    }
+
+    // ring and butterfly: chunk c has one final owner who folds all N operands.
+    //   butterfly (AllreduceAlgos.cpp:151-180): owner c; order own, then peers ascending.
+    //   ring      (AllreduceAlgos.cpp:62-75)  : owner (c-1) mod N; order c, c+1, ..., owner.
+    const bool ring = r->algo == MCCLX_ALGO_RING;
+    Chunks c((int64_t)r->numel, 1, N);  // element offsets; bytes derived per buffer
+    auto owner_of = [&](int chunk) { return ring ? (chunk - 1 + N) % N : chunk; };
+    auto order_of = [&](int chunk, int j) {  // rank of the j-th operand
+        if (ring) return (chunk + j) % N;
+        if (j == 0) return chunk;
+        return (j - 1 < chunk) ? j - 1 : j;  // ascending peers, skipping the owner
+    };
+
+    if (L.wire) {
+        // every rank encodes what it sends: all chunks except the one it owns
+        mcclx_plan e = base_plan(r, L, 1);
+        e.io = MCCLX_IO_OWN_FIRST_F32;
+        e.op = MCCLX_SUM;
+        e.scale_mode = MCCLX_SCALE_NONE;
+        for (int q = 0; q < N; ++q)
+            for (int ch = 0; ch < N; ++ch) {
+                if (owner_of(ch) == q || c[ch].elem_count == 0) continue;
+                mcclx_seg s = z;
+                s.wire_out = at(wire_of(q), (uint64_t)c[ch].elem_start * 2);
+                s.in[0] = at(r->tensors[q], (uint64_t)c[ch].elem_start * 4);
+                s.count = (uint64_t)c[ch].elem_count;
+                segs.push_back(s);
+            }
+        if (!segs.empty()) TRY(mcclx_fold_batched(ctx, &e, segs.data(), (uint32_t)segs.size()));
+        segs.clear();
+    }
+
+    mcclx_plan p = base_plan(r, L, N);
+    if (L.wire) p.io = ring ? MCCLX_IO_OWN_LAST_F32 : MCCLX_IO_OWN_FIRST_F32;
+    for (int ch = 0; ch < N; ++ch) {
+        if (c[ch].elem_count == 0) continue;
+        int o = owner_of(ch);
+        mcclx_seg s = z;
+        s.count = (uint64_t)c[ch].elem_count;
+        s.out = at(r->tensors[o], (uint64_t)c[ch].elem_start * ts);
+        if (L.wire) s.wire_out = at(wire_of(o), (uint64_t)c[ch].elem_start * 2);
+        for (int j = 0; j < N; ++j) {
+            int q = order_of(ch, j);
+            if (L.wire && q != o)
+                s.in[j] = at(wire_of(q), (uint64_t)c[ch].elem_start * es);
+            else
+                s.in[j] = at(r->tensors[q], (uint64_t)c[ch].elem_start * ts);
+        }
+        segs.push_back(s);
+    }
+    TRY(fold_any(ctx, p, segs));
+    segs.clear();
+
+    // allgather leg (AllreduceAlgos.cpp:77-86,185-200): every other rank gets
+    // the owner's reduced chunk; with the wire codec it arrives as bf16 and is
+    // cast on arrival (ProcessGroupMCCL.cpp:179-183).
+    if (L.wire) {
+        mcclx_plan d = base_plan(r, L, 1);
+        d.io = MCCLX_IO_OUT_F32;
+        d.op = MCCLX_SUM;
+        d.scale_mode = MCCLX_SCALE_NONE;
+        for (int ch = 0; ch < N; ++ch) {
+            if (c[ch].elem_count == 0) continue;
+            int o = owner_of(ch);
+            for (int q = 0; q < N; ++q) {
+                if (q == o) continue;
+                mcclx_seg s = z;
+                s.out = at(r->tensors[q], (uint64_t)c[ch].elem_start * 4);
+                s.in[0] = at(wire_of(o), (uint64_t)c[ch].elem_start * 2);
+                s.count = (uint64_t)c[ch].elem_count;
+                segs.push_back(s);
+            }
+        }
+        if (!segs.empty()) TRY(mcclx_fold_batched(ctx, &d, segs.data(), (uint32_t)segs.size()));
+    } else {
+        for (int ch = 0; ch < N; ++ch) {
+            int o = owner_of(ch);
+            for (int q = 0; q < N; ++q)
+                if (q != o)
+                    TRY(mcclx_copy(ctx, at(r->tensors[q], (uint64_t)c[ch].elem_start * ts),
+                                   at(r->tensors[o], (uint64_t)c[ch].elem_start * ts),
+                                   (uint64_t)c[ch].elem_count * ts));
+        }
+    }
+    return MCCLX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mcclx_chunkize(int64_t numel, uint64_t elem_size, int world, mcclx_chunk* out) {
+    if (world < 1 || numel < 0 || !out) return bad("chunkize: bad argument");
+    const int64_t per = (numel + world - 1) / world;  // AllreduceAlgos.cpp:23
+    for (int i = 0; i < world; ++i) {
+        int64_t lo = (int64_t)i * per, hi = lo + per;
+        lo = lo < numel ? lo : numel;
+        hi = hi < numel ? hi : numel;
+        out[i] = mcclx_chunk{lo, hi - lo, (uint64_t)lo * elem_size, (uint64_t)(hi - lo) * elem_size};
+    }
+    return MCCLX_OK;
+}
+
+int mcclx_select_algo(const char* env_algo, int64_t tree_below, uint64_t wire_nbytes,
+                      int64_t numel, int world) {
+    std::string alg = env_algo ? env_algo : "auto";  // ProcessGroupMCCL.cpp:134-135
+    int algo = MCCLX_ALGO_TREE;                     // any unknown name runs the tree (:173-176)
+    if (alg == "auto") {
+        uint64_t below = tree_below < 0 ? 256ull * 1024 : (uint64_t)tree_below;  // :137-139
+        algo = wire_nbytes <= below ? MCCLX_ALGO_TREE : MCCLX_ALGO_RING;        // :140
+    } else if (alg == "ring") {
+        algo = MCCLX_ALGO_RING;
+    } else if (alg == "butterfly") {
+        algo = MCCLX_ALGO_BUTTERFLY;
+    }
+    if (algo == MCCLX_ALGO_RING && numel < world) algo = MCCLX_ALGO_TREE;  // :143
+    if (algo == MCCLX_ALGO_BUTTERFLY && (world < 2 || numel < world)) algo = MCCLX_ALGO_TREE;  // :144-145
+    return algo;
+}
+
+uint64_t mcclx_replay_workspace_bytes(const mcclx_replay* r) {
+    if (!r || r->world < 1) return 0;
+    return layout_of(r).total;
+}
+
+int mcclx_allreduce_replay(mcclx_ctx* ctx, const mcclx_replay* r) {
+    if (!ctx || !r || !r->tensors) return bad("replay: null argument");
+    if (r->world < 1 || r->reserved != 0) return bad("replay: bad world");
+    if (r->algo < MCCLX_ALGO_RING || r->algo > MCCLX_ALGO_BUTTERFLY) return bad("replay: bad algo");
+    if (r->mode != MCCLX_REPLAY_STEPWISE && r->mode != MCCLX_REPLAY_FUSED) return bad("replay: bad mode");
+    if (r->op < MCCLX_SUM || r->op > MCCLX_MAX) {
+        // surfaces "Unsupported ReduceOp: n" through the kernel layer
+        return mcclx_reduce(ctx, r->tensors[0], r->tensors[0], r->dtype, 0, r->op);
+    }
+    if (r->world == 1) return MCCLX_OK;  // ProcessGroupMCCL.cpp:107
+    if (r->numel == 0) return bad("replay: empty tensor");  // TensorChecks.hpp:31-34
+    // AllreduceAlgos.cpp:55,137
+    if (r->algo != MCCLX_ALGO_TREE && r->numel < (uint64_t)r->world) return bad("numel must be >= world");
+    for (int i = 0; i < r->world; ++i)
+        if (!r->tensors[i]) return bad("replay: null tensor");
+    Layout L = layout_of(r);
+    if (L.total > 0 && (!r->workspace || r->workspace_bytes < L.total)) return bad("workspace too small");
+
+    bool fused = r->mode == MCCLX_REPLAY_FUSED && r->world <= MCCLX_MAX_INPUTS;
+    // the binomial tree of the binary-only kernels (MIN/MAX/PRODUCT, fp16) has
+    // no fused form
+    // Also, a chain of binary launches into `out` needs out to be operand 0
+    // (butterfly); the ring's owner is the LAST operand, and the wire codec
+    // mixes fp32 and bf16 operands, which only the SUM fold handles.
+    bool binary_only = (r->op != MCCLX_SUM && r->op != MCCLX_AVG) || L.wdtype == MCCLX_F16;
+    if (fused && binary_only && r->world > 2 &&
+        (r->algo != MCCLX_ALGO_BUTTERFLY || L.wire))
+        fused = false;
+    if (fused && binary_only && L.wire) fused = false;
+    if (!fused) {
+        mcclx_replay s = *r;
+        s.mode = MCCLX_REPLAY_STEPWISE;
+        Layout Ls = layout_of(&s);
+        if (Ls.total > 0 && (!r->workspace || r->workspace_bytes < Ls.total)) return bad("workspace too small");
+        return replay_stepwise(ctx, &s, Ls);
+    }
+    return replay_fused(ctx, r, L);
+}
+
+int mcclx_reduce_scatter_replay(mcclx_ctx* ctx, int world, void* const* outs,
+                                const void* const* ins, int dtype, uint64_t chunk_numel, int op,
+                                int mode, int acc) {
+    if (!ctx || !outs || !ins || world < 1) return bad("reduce_scatter: bad argument");
+    const uint64_t cb = chunk_numel * esize(dtype);
+    if (world == 1) return mcclx_copy(ctx, outs[0], ins[0], cb);  // ProcessGroupMCCL.cpp:333-337
+    bool binary_only = (op != MCCLX_SUM && op != MCCLX_AVG) || dtype == MCCLX_F16;
+    bool fused = mode == MCCLX_REPLAY_FUSED && world <= MCCLX_MAX_INPUTS;
+    if (!fused) {
+        for (int r = 0; r < world; ++r) {  // :357, :378-386
+            TRY(mcclx_copy(ctx, outs[r], at(ins[r], (uint64_t)r * cb), cb));
+            for (int p = 0; p < world; ++p)
+                if (p != r) TRY(mcclx_reduce(ctx, outs[r], at(ins[p], (uint64_t)r * cb), dtype, chunk_numel, op));
+            if (op == MCCLX_AVG)
+                TRY(mcclx_scale(ctx, outs[r], dtype, chunk_numel, 1.0 / (double)world, MCCLX_SCALE_TENSOR));
+        }
+        return MCCLX_OK;
+    }
+    mcclx_plan p;
+    memset(&p, 0, sizeof p);
+    p.dtype = dtype;
+    p.io = MCCLX_IO_PURE;
+    p.k = world;
+    p.topo = MCCLX_TOPO_FOLD;
+    p.op = op;
+    p.acc = acc;
+    p.scale_mode = (op == MCCLX_AVG) ? MCCLX_SCALE_TENSOR : MCCLX_SCALE_NONE;  // metal_scale_inplace
+    p.scale = 1.0 / (double)world;
+    std::vector<mcclx_seg> segs((size_t)world);
+    for (int r = 0; r < world; ++r) {
+        memset(&segs[r], 0, sizeof(mcclx_seg));
+        segs[r].out = outs[r];
+        segs[r].count = chunk_numel;
+        segs[r].in[0] = at(ins[r], (uint64_t)r * cb);  // own share first (:357)
+        int j = 1;
+        for (int q = 0; q < world; ++q)
+            if (q != r) segs[r].in[j++] = at(ins[q], (uint64_t)r * cb);  // ascending peers (:379-383)
+    }
+    if (binary_only) p.acc = MCCLX_ACC_STEP;
+    return fold_any(ctx, p, segs);
+}
+
+int mcclx_allgather_replay(mcclx_ctx* ctx, int world, void* const* outs, const void* const* ins,
+                           uint64_t chunk_nbytes) {
+    if (!ctx || !outs || !ins || world < 1) return bad("allgather: bad argument");
+    for (int r = 0; r < world; ++r)
+        for (int p = 0; p < world; ++p)  // ProcessGroupMCCL.cpp:256-270
+            TRY(mcclx_copy(ctx, at(outs[r], (uint64_t)p * chunk_nbytes), ins[p], chunk_nbytes));
+    return MCCLX_OK;
+}
+
+}  // extern "C"

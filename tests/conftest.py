@@ -3,9 +3,13 @@ import sys
 
 import pytest
 
+# libmcclx checks every launch's pointers against their allocations when this is set
+os.environ.setdefault("MCCLX_VALIDATE", "1")
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-if ROOT not in sys.path:
-    sys.path.insert(0, ROOT)
+for p in (ROOT, os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
 
 
 def pytest_configure(config):

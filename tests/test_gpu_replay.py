@@ -1,0 +1,206 @@
+"""GPU parity of the chunk scheduler: the N-virtual-rank replay of ring / tree /
+butterfly allreduce, reduce_scatter and allgather (STEPWISE = the reference's
+launches one by one, FUSED = one multi-input pass per chunk) against the
+oracle's message-by-message replay of the reference."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from oracle.oracle import F32, F16, BF16, SUM, AVG, PRODUCT, MIN, MAX, RING, TREE, BUTTERFLY
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K():
+    from mccl_amd import kernels
+    kernels.hip_kernels_init(0)
+    return kernels
+
+
+@pytest.fixture(scope="module")
+def H():
+    from mccl_amd import harness
+    return harness
+
+
+@pytest.fixture(scope="module")
+def U():
+    import gpu_util
+    return gpu_util
+
+
+STEPWISE, FUSED = 0, 1
+
+
+def run_case(H, U, algo, world, dtype, op, wire, mode, numel, seed, specials=False):
+    rng = np.random.default_rng(seed)
+    xs = [U.rand_values(rng, numel, dtype, scale=10.0 ** rng.integers(-3, 2), specials=specials)
+          for _ in range(world)]
+    want = [x.copy() for x in xs]
+    rc = orc.allreduce(algo, want, dtype, op) if not wire else \
+        orc.pg_allreduce(want, dtype, op, wire_bf16=True, env_algo={RING: "ring", TREE: "tree", BUTTERFLY: "butterfly"}[algo])[0]
+    assert rc == 0
+    d = [U.to_dev(x, dtype) for x in xs]
+    H.allreduce_replay(d, op, algo, wire_bf16=wire, mode=mode)
+    for r in range(world):
+        if dtype == F16:
+            assert np.array_equal(U.bits(d[r]), want[r]), (algo, world, r)
+        else:
+            U.assert_same_bits(d[r], want[r], dtype, f"algo={algo} world={world} rank={r} op={op} wire={wire} mode={mode}")
+
+
+@pytest.mark.parametrize("algo", [RING, TREE, BUTTERFLY])
+@pytest.mark.parametrize("world", [2, 3, 4, 5, 8])
+@pytest.mark.parametrize("mode", [STEPWISE, FUSED])
+@pytest.mark.parametrize("dtype,wire", [(F32, False), (BF16, False), (F32, True)])
+def test_allreduce_sum_avg(H, U, algo, world, mode, dtype, wire):
+    for op in (SUM, AVG):
+        for numel in (world, 1237, 40009):   # numel == world: one element per chunk
+            run_case(H, U, algo, world, dtype, op, wire, mode, numel, seed=world * 100 + algo * 10 + op,
+                     specials=(numel > 1000 and dtype != F16))
+
+
+@pytest.mark.parametrize("algo", [RING, TREE, BUTTERFLY])
+@pytest.mark.parametrize("op", [PRODUCT, MIN, MAX])
+@pytest.mark.parametrize("mode", [STEPWISE, FUSED])
+def test_allreduce_other_ops_and_fp16(H, U, algo, op, mode):
+    for world in (2, 3, 4):
+        for dtype, wire in ((F32, False), (BF16, False), (F16, False), (F32, True)):
+            run_case(H, U, algo, world, dtype, op, wire, mode, 5003, seed=world + op)
+    run_case(H, U, algo, 3, F16, SUM, False, mode, 5003, seed=1)
+    run_case(H, U, algo, 3, F16, AVG, False, mode, 5003, seed=2)
+
+
+@pytest.mark.parametrize("algo", [RING, TREE, BUTTERFLY])
+def test_wide_world_falls_back_to_stepwise(H, U, algo):
+    run_case(H, U, algo, 11, F32, SUM, True, FUSED, 2003, seed=11)
+    run_case(H, U, algo, 16, BF16, AVG, False, FUSED, 2003, seed=16)
+
+
+def test_tree_with_fewer_elements_than_ranks(H, U):  # ProcessGroupMCCL.cpp:143-145 -> tree
+    for mode in (STEPWISE, FUSED):
+        run_case(H, U, TREE, 5, F32, SUM, False, mode, 3, seed=3)
+        run_case(H, U, TREE, 4, F32, AVG, True, mode, 1, seed=4)
+
+
+def test_preconditions(H):
+    from mccl_amd import MCCLError
+    t = [torch.ones(2, device="cuda") for _ in range(3)]
+    for algo in (RING, BUTTERFLY):
+        with pytest.raises(MCCLError, match="numel must be >= world"):   # AllreduceAlgos.cpp:55,137
+            H.allreduce_replay(t, SUM, algo)
+    with pytest.raises(MCCLError, match="Unsupported ReduceOp: 5"):
+        H.allreduce_replay(t, 5, TREE)
+    with pytest.raises(MCCLError, match="empty tensor list"):
+        H.allreduce_replay([], SUM, TREE)
+    one = [torch.full((4,), 7.0, device="cuda")]
+    H.allreduce_replay(one, AVG, RING)                                   # world == 1: no-op (PG.cpp:107)
+    assert torch.equal(one[0], torch.full((4,), 7.0, device="cuda"))
+
+
+def test_env_semantics(H, U, monkeypatch):
+    """MCCL_ALLREDUCE_ALGO / MCCL_TREE_BELOW / MCCL_WIRE_DTYPE are re-read per call."""
+    rng = np.random.default_rng(9)
+
+    def go(numel, world=3, dtype=F32):
+        xs = [U.rand_values(rng, numel, dtype) for _ in range(world)]
+        d = [U.to_dev(x, dtype) for x in xs]
+        used = H.allreduce(d, "sum")
+        return xs, d, used
+
+    for k in ("MCCL_ALLREDUCE_ALGO", "MCCL_TREE_BELOW", "MCCL_WIRE_DTYPE"):
+        monkeypatch.delenv(k, raising=False)
+    assert go(65536)[2] == TREE            # 262144 B <= default threshold (inclusive)
+    assert go(65537)[2] == RING
+    monkeypatch.setenv("MCCL_TREE_BELOW", "1000")
+    assert go(300)[2] == RING and go(250)[2] == TREE
+    monkeypatch.setenv("MCCL_WIRE_DTYPE", "bf16")
+    assert go(500)[2] == TREE              # threshold applies to the bf16 byte size
+    assert go(500, dtype=BF16)[2] == TREE and go(501, dtype=BF16)[2] == RING
+    monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "butterfly")
+    xs, d, used = go(999)
+    assert used == BUTTERFLY
+    want = [x.copy() for x in xs]
+    assert orc.pg_allreduce(want, F32, SUM, wire_bf16=True, env_algo="butterfly", tree_below=1000) == (0, BUTTERFLY)
+    U.assert_same_bits(d[1], want[1], F32, "env butterfly + wire")
+    assert go(2)[2] == TREE                # numel < world
+    monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "nonsense")
+    assert go(100000)[2] == TREE
+    monkeypatch.setenv("MCCL_WIRE_DTYPE", "fp16")   # only "bf16" switches the codec on
+    monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "ring")
+    xs, d, used = go(999)
+    want = [x.copy() for x in xs]; orc.allreduce(RING, want, F32, SUM)
+    U.assert_same_bits(d[0], want[0], F32, "no wire")
+
+
+@pytest.mark.parametrize("world", [2, 3, 8, 10])
+@pytest.mark.parametrize("dtype", [F32, BF16, F16])
+@pytest.mark.parametrize("mode", [STEPWISE, FUSED])
+def test_reduce_scatter_allgather(H, U, world, dtype, mode):
+    rng = np.random.default_rng(world)
+    CH = 4099
+    for op in (SUM, AVG, MIN, MAX, PRODUCT):
+        ins = [U.rand_values(rng, CH * world, dtype) for _ in range(world)]
+        want = [np.zeros(CH, dtype=ins[0].dtype) for _ in range(world)]
+        assert orc.reduce_scatter(want, ins, dtype, op) == 0
+        din = [U.to_dev(x, dtype) for x in ins]
+        dout = [torch.empty(CH, dtype=din[0].dtype, device="cuda") for _ in range(world)]
+        H.reduce_scatter_replay(dout, din, op, mode=mode)
+        for r in range(world):
+            if dtype == F16:
+                assert np.array_equal(U.bits(dout[r]), want[r])
+            else:
+                U.assert_same_bits(dout[r], want[r], dtype, f"reduce_scatter op={op} rank={r}")
+    # in place: out is the rank's own slice of its input (tests/collectives/test_reduce_scatter.py:24-29)
+    ins = [U.rand_values(rng, CH * world, dtype) for _ in range(world)]
+    want = [np.zeros(CH, dtype=ins[0].dtype) for _ in range(world)]
+    orc.reduce_scatter(want, ins, dtype, SUM)
+    din = [U.to_dev(x, dtype) for x in ins]
+    dout = [din[r].narrow(0, r * CH, CH) for r in range(world)]
+    H.reduce_scatter_replay(dout, din, SUM, mode=mode)
+    for r in range(world):
+        if dtype == F16:
+            assert np.array_equal(U.bits(dout[r]), want[r])
+        else:
+            U.assert_same_bits(dout[r], want[r], dtype, "in place")
+    # allgather of the results (tests/collectives/allgather.py)
+    gout = [torch.empty(CH * world, dtype=din[0].dtype, device="cuda") for _ in range(world)]
+    H.allgather_replay(gout, [o.contiguous() for o in dout])
+    cat = np.concatenate([U.bits(o) for o in dout])
+    for g in gout:
+        assert np.array_equal(U.bits(g), cat)
+
+
+def test_reduce_scatter_reference_vectors(H, U):
+    """tests/collectives/test_reduce_scatter.py:14-44: value (p+1)*10+rank, CHUNK=32."""
+    world, CH = 4, 32
+    for dtype, tdt in ((F32, torch.float32), (BF16, torch.bfloat16), (F16, torch.float16)):
+        ins = [torch.cat([torch.full((CH,), float((p + 1) * 10 + r), dtype=tdt, device="cuda")
+                          for p in range(world)]) for r in range(world)]
+        outs = [torch.empty(CH, dtype=tdt, device="cuda") for _ in range(world)]
+        H.reduce_scatter_replay(outs, ins, "sum")
+        for r in range(world):
+            exp = sum((r + 1) * 10 + q for q in range(world))
+            assert torch.allclose(outs[r].float().cpu(), torch.full((CH,), float(exp)), rtol=1e-2, atol=1e-2)
+        H.reduce_scatter_replay(outs, ins, "max")
+        for r in range(world):
+            assert torch.equal(outs[r].float().cpu(), torch.full((CH,), float((r + 1) * 10 + world - 1)))
+
+
+def test_f32acc_reduce_scatter_variant(H, U):
+    """The fp32-accumulate mode (not the reference) equals its own oracle and
+    stays within one bf16 ulp of the exact sum."""
+    rng = np.random.default_rng(8)
+    world, CH = 8, 10007
+    ins = [U.rand_values(rng, CH * world, BF16, scale=1e-2) for _ in range(world)]
+    want = [np.zeros(CH, dtype=np.uint16) for _ in range(world)]
+    orc.reduce_scatter_f32acc(want, ins, SUM)
+    din = [U.to_dev(x, BF16) for x in ins]
+    dout = [torch.empty(CH, dtype=torch.bfloat16, device="cuda") for _ in range(world)]
+    H.reduce_scatter_replay(dout, din, SUM, mode=FUSED, acc=1)
+    for r in range(world):
+        assert np.array_equal(U.bits(dout[r]), want[r])
