@@ -125,6 +125,7 @@ def main():
         return ms_dev, (time.perf_counter() - t0) * 1e3
 
     def measure(seg_fn, steps, warmup):
+        torch.cuda.synchronize()  # inputs made by torch ops are complete before the queue reads them
         gw = record(max(1, warmup), seg_fn)
         gk = record(steps, seg_fn)
         q.graph_launch(gw)

@@ -201,6 +201,27 @@ def make_plan(dtype, k, io=L.IO_PURE, topo=L.TOPO_FOLD, op=L.SUM, acc=L.ACC_STEP
 
 
 # ---- tensor variants (MetalKernels.hpp:14-43) ------------------------------
+#
+# Tensors are produced and consumed on torch's current stream, the kernels run
+# on the reduce queue: each tensor variant makes the queue wait for torch's
+# stream before the launch and torch's stream wait for the queue after it
+# (two device-side event waits, the host is never blocked).  The reference
+# reaches the same ordering with a blocking mps_stream_sync() before and
+# mccl_queue_drain() after (ProcessGroupMCCL.cpp:172,178).  The *_view variants
+# take raw addresses and leave the ordering to the caller, as the reference's do.
+
+class _ordered:
+    def __init__(self, q: "ReduceQueue"):
+        self.q = q
+
+    def __enter__(self):
+        self.q.wait_torch_stream()
+        return self.q
+
+    def __exit__(self, *exc):
+        self.q.torch_stream_wait()
+        return False
+
 
 def hip_reduce_op(dst: torch.Tensor, src: torch.Tensor, op, queue=None) -> torch.Tensor:
     """dst (op)= src.  metal_reduce_op, MetalKernels.mm:530-550."""
@@ -208,8 +229,10 @@ def hip_reduce_op(dst: torch.Tensor, src: torch.Tensor, op, queue=None) -> torch
     _check_tensor(dst, "reduce_op")
     _check_tensor(src, "reduce_op")
     _check_same(dst, src)
-    L.check(L.lib().mcclx_reduce(q.handle, dst.data_ptr(), src.data_ptr(), dtype_code(dst),
-                                 dst.numel(), op_code(op)))
+    code = dtype_code(dst)
+    with _ordered(q):
+        L.check(L.lib().mcclx_reduce(q.handle, dst.data_ptr(), src.data_ptr(), code, dst.numel(),
+                                     op_code(op)))
     return dst
 
 
@@ -233,8 +256,10 @@ def hip_scale_inplace(buf: torch.Tensor, scale: float, queue=None) -> torch.Tens
     """buf *= scale, tensor-variant constant.  metal_scale_inplace, MetalKernels.mm:365-405."""
     q = _q(queue)
     _check_tensor(buf, "scale_inplace")
-    L.check(L.lib().mcclx_scale(q.handle, buf.data_ptr(), dtype_code(buf), buf.numel(), float(scale),
-                                L.SCALE_TENSOR))
+    code = dtype_code(buf)
+    with _ordered(q):
+        L.check(L.lib().mcclx_scale(q.handle, buf.data_ptr(), code, buf.numel(), float(scale),
+                                    L.SCALE_TENSOR))
     return buf
 
 
@@ -244,8 +269,10 @@ def hip_accumulate_and_scale(dst, src, scale: float, queue=None) -> torch.Tensor
     _check_tensor(dst, "accumulate_and_scale")
     _check_tensor(src, "accumulate_and_scale")
     _check_same(dst, src)
-    L.check(L.lib().mcclx_accumulate_scale(q.handle, dst.data_ptr(), src.data_ptr(), dtype_code(dst),
-                                           dst.numel(), float(scale)))
+    code = dtype_code(dst)
+    with _ordered(q):
+        L.check(L.lib().mcclx_accumulate_scale(q.handle, dst.data_ptr(), src.data_ptr(), code,
+                                               dst.numel(), float(scale)))
     return dst
 
 
@@ -296,7 +323,8 @@ def encode_bf16(src: torch.Tensor, out: Optional[torch.Tensor] = None, queue=Non
         raise MCCLError("[MCCL] encode_bf16 expects a float32 tensor")
     if out is None:
         out = torch.empty(src.shape, dtype=torch.bfloat16, device=src.device)
-    L.check(L.lib().mcclx_encode_bf16(q.handle, out.data_ptr(), src.data_ptr(), src.numel()))
+    with _ordered(q):
+        L.check(L.lib().mcclx_encode_bf16(q.handle, out.data_ptr(), src.data_ptr(), src.numel()))
     return out
 
 
@@ -308,5 +336,6 @@ def decode_bf16(src: torch.Tensor, out: Optional[torch.Tensor] = None, queue=Non
         raise MCCLError("[MCCL] decode_bf16 expects a bfloat16 tensor")
     if out is None:
         out = torch.empty(src.shape, dtype=torch.float32, device=src.device)
-    L.check(L.lib().mcclx_decode_bf16(q.handle, out.data_ptr(), src.data_ptr(), src.numel()))
+    with _ordered(q):
+        L.check(L.lib().mcclx_decode_bf16(q.handle, out.data_ptr(), src.data_ptr(), src.numel()))
     return out

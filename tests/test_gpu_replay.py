@@ -23,7 +23,8 @@ def K():
 
 @pytest.fixture(scope="module")
 def H():
-    from mccl_amd import harness
+    from mccl_amd import harness, kernels
+    kernels.hip_kernels_init(0)
     return harness
 
 
