@@ -31,6 +31,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+CAL_BYTES = 64 << 20   # size of the calibration copy
 
 
 def parse():
@@ -79,6 +80,14 @@ def main():
         ws = [K.encode_bf16(t, queue=q) for t in ts]
         tensors.append(ts)
         wires.append(ws)
+    q.drain()
+
+    # A plain copy of known size (64 MiB in, 64 MiB out), 5 launches: the reference
+    # dispatches the memory counters (FETCH_SIZE / WRITE_SIZE) are scaled by.
+    cal = torch.empty(2 * CAL_BYTES, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    for _ in range(5):
+        q.copy(cal.data_ptr() + CAL_BYTES, cal.data_ptr(), CAL_BYTES)
     q.drain()
 
     plan = K.make_plan(L.BF16, world, io=L.IO_OWN_FIRST_F32, op=L.SUM, scale_mode=L.SCALE_VIEW, scale=scale)

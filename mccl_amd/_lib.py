@@ -10,7 +10,8 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libmcclx.so")
+# MCCLX_LIBRARY names a differently built libmcclx.so (tuning builds); default: the in-tree one.
+LIB_PATH = os.environ.get("MCCLX_LIBRARY") or os.path.join(HERE, "libmcclx.so")
 
 MAX_INPUTS = 8
 

@@ -11,12 +11,18 @@
 //   N-1 binary launches + casts + scale of one schedule k=N, any io, one pass
 //
 // The work is HBM-bound streaming (0.1-0.25 flop/byte), so there is no MFMA
-// and no LDS: every lane moves 16-byte packets (global_load/store_dwordx4),
-// a wavefront covers 1 KiB of each stream per packet, all loads of an
-// iteration are issued before the first dependent ALU op, and the arithmetic
-// (bf16 round-to-nearest-even in integer ops) hides under the memory time.
-// Pointers only need element alignment: gfx950 global accesses are
-// alignment-agnostic and the compiler is told so through under-aligned types.
+// and no LDS.  Consecutive lanes take consecutive packets of E elements, so one
+// wavefront instruction covers one contiguous span of every stream: E = 4 when
+// any stream is fp32 (fp32: global_load/store_dwordx4 = 1 KiB per wavefront,
+// 16-bit peers: dwordx2 = 512 B), E = 8 when every stream is 16-bit (dwordx4).
+// All loads of an iteration are issued before the first dependent ALU op and
+// the arithmetic (bf16 round-to-nearest-even) hides under the memory time.
+// Accesses carry the non-temporal hint: every byte is touched exactly once.
+// Pointers only need element alignment (gfx950 global accesses are
+// alignment-agnostic and the compiler is told so through under-aligned
+// types); a scalar head peel moves the packet grid onto a 128-byte boundary of
+// the output, which also aligns the inputs whenever all buffers share the
+// chunk's element offset.
 //
 // Numerics: IEEE fp32 add/mul (no contraction, denormals kept), rounded to the
 // arithmetic dtype after EVERY operation in MCCLX_ACC_STEP mode -- the
@@ -31,13 +37,30 @@
 namespace mcclx {
 namespace {
 
-constexpr int kBlock = 256;   // 4 wavefronts of 64
-constexpr int kPack = 8;      // elements per packet: 16 B of bf16/f16, 32 B of fp32
+// Build-time tuning knobs (defaults are the measured best on MI355X).
+#ifndef MCCLX_TUNE_BLOCK
+#define MCCLX_TUNE_BLOCK 256
+#endif
+#ifndef MCCLX_TUNE_U
+#define MCCLX_TUNE_U 0  // 0: derive from the register budget of the plan
+#endif
+#ifndef MCCLX_TUNE_NT_LOAD
+#define MCCLX_TUNE_NT_LOAD 1
+#endif
+#ifndef MCCLX_TUNE_NT_STORE
+#define MCCLX_TUNE_NT_STORE 1
+#endif
+#ifndef MCCLX_TUNE_HWCVT
+#define MCCLX_TUNE_HWCVT 1  // 1: v_cvt_pk_bf16_f32 + NaN fix-up; 0: integer rounding
+#endif
+#ifndef MCCLX_TUNE_PEEL
+#define MCCLX_TUNE_PEEL 1   // scalar head peel up to the output's 128-byte boundary
+#endif
+
+constexpr int kBlock = MCCLX_TUNE_BLOCK;  // wavefronts of 64 lanes
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // Under-aligned views: element alignment is all the kernels may assume.
-struct __attribute__((packed, aligned(2))) Raw16 { u32x4 q; };
-struct __attribute__((packed, aligned(4))) Raw32 { u32x4 lo; u32x4 hi; };
 
 // Every operand lives in global memory (HBM or host memory mapped into the
 // device).  Pointers that reach a kernel through a descriptor table are
@@ -50,15 +73,36 @@ template <class T> __device__ __forceinline__ const MCCLX_GLOBAL T* gptr(const v
 template <class T> __device__ __forceinline__ MCCLX_GLOBAL T* gptr(void* p) {
     return (MCCLX_GLOBAL T*)p;
 }
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+typedef u32x2 u32x2_a2 __attribute__((aligned(2)));
+// Loads and stores of one packet through the under-aligned pointer types
+// (macros, so the typedef's alignment stays attached to the access).
+#if MCCLX_TUNE_NT_LOAD
+#define MCCLX_LDG(p) __builtin_nontemporal_load(p)
+#else
+#define MCCLX_LDG(p) (*(p))
+#endif
+#if MCCLX_TUNE_NT_STORE
+#define MCCLX_STG(p, v) __builtin_nontemporal_store((v), (p))
+#else
+#define MCCLX_STG(p, v) (*(p) = (v))
+#endif
 
 // ---------------------------------------------------------------- rounding
 
 // fp32 -> bf16 round-to-nearest-even, NaN -> 0x7FC0, result kept as the fp32
 // whose low half is zero (torch/headeronly/util/BFloat16.h:100-114).
 __device__ __forceinline__ uint32_t bf16_round_bits(float x) {
+#if MCCLX_TUNE_HWCVT
+    uint32_t r = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)x) << 16;
+    return (x != x) ? 0x7FC00000u : r;
+#else
     uint32_t u = __float_as_uint(x);
     uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
     return ((u & 0x7FFFFFFFu) > 0x7F800000u) ? 0x7FC00000u : r;
+#endif
 }
 
 template <int W> struct Num;  // arithmetic dtype traits
@@ -100,49 +144,48 @@ template <int W_, int IO_, int K_, int TOPO_, int OP_, int ACC_>
 struct Cfg {
     static constexpr int W = W_, IO = IO_, K = K_, TOPO = TOPO_, OP = OP_, ACC = ACC_;
     static constexpr bool kOutF32 = (IO != MCCLX_IO_PURE);
+    // elements per packet: 4 as soon as one stream (operand or output) is fp32
+    static constexpr int E = (W == MCCLX_F32 || IO != MCCLX_IO_PURE) ? 4 : 8;
     __host__ __device__ static constexpr bool in_is_f32(int k) {
         return W == MCCLX_F32 || (IO == MCCLX_IO_OWN_FIRST_F32 && k == 0) ||
                (IO == MCCLX_IO_OWN_LAST_F32 && k == K - 1);
     }
     __host__ __device__ static constexpr int regs_per_pack() {
         int r = 0;
-        for (int k = 0; k < K; ++k) r += in_is_f32(k) ? 8 : 4;
+        for (int k = 0; k < K; ++k) r += (in_is_f32(k) || E == 8) ? 4 : 2;
         return r;
     }
-    // packets in flight per lane per iteration: keep raw loads near 64 registers
-    static constexpr int U = (TOPO == MCCLX_TOPO_BINOMIAL) ? 1
-                             : (64 / regs_per_pack() >= 4 ? 4 : 64 / regs_per_pack() >= 2 ? 2 : 1);
+    // packets in flight per lane per iteration
+    static constexpr int U = MCCLX_TUNE_U ? MCCLX_TUNE_U
+                             : (TOPO == MCCLX_TOPO_BINOMIAL) ? 1
+                             : (32 / regs_per_pack() >= 2 ? 2 : 1);
 };
 
-struct RawPack { u32x4 a; u32x4 b; };  // b only used by fp32 packets
+typedef u32x4 RawPack;  // one packet of one operand: 16 B, or 8 B in .xy (16-bit operand, E = 4)
 
 template <class C, int k>
 __device__ __forceinline__ RawPack load_raw(const void* p, uint64_t pack) {
-    RawPack r;
     if constexpr (C::in_is_f32(k)) {
-        const MCCLX_GLOBAL Raw32* q = gptr<Raw32>(static_cast<const float*>(p) + pack * kPack);
-        r.a = q->lo; r.b = q->hi;
+        return MCCLX_LDG(gptr<u32x4_a4>(static_cast<const float*>(p) + pack * C::E));
+    } else if constexpr (C::E == 8) {
+        return MCCLX_LDG(gptr<u32x4_a2>(static_cast<const uint16_t*>(p) + pack * C::E));
     } else {
-        const MCCLX_GLOBAL Raw16* q = gptr<Raw16>(static_cast<const uint16_t*>(p) + pack * kPack);
-        r.a = q->q; r.b = r.a;
+        u32x2 h = MCCLX_LDG(gptr<u32x2_a2>(static_cast<const uint16_t*>(p) + pack * C::E));
+        return u32x4{h.x, h.y, 0u, 0u};
     }
-    return r;
 }
 
 // Operand k of one packet as 8 floats holding W-representable values.
 template <class C, int k>
-__device__ __forceinline__ void decode(const RawPack& r, float (&v)[kPack]) {
+__device__ __forceinline__ void decode(const RawPack& r, float (&v)[C::E]) {
     if constexpr (C::in_is_f32(k)) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            v[j] = Num<C::W>::rnd(__uint_as_float(r.a[j]));      // own fp32 -> wire value
-            v[4 + j] = Num<C::W>::rnd(__uint_as_float(r.b[j]));
-        }
+        for (int j = 0; j < 4; ++j) v[j] = Num<C::W>::rnd(__uint_as_float(r[j]));  // own fp32 -> wire value
     } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            v[2 * j] = Num<C::W>::dec(r.a[j] & 0xFFFFu);
-            v[2 * j + 1] = Num<C::W>::dec(r.a[j] >> 16);
+        for (int j = 0; j < C::E / 2; ++j) {
+            v[2 * j] = Num<C::W>::dec(r[j] & 0xFFFFu);
+            v[2 * j + 1] = Num<C::W>::dec(r[j] >> 16);
         }
     }
 }
@@ -173,68 +216,74 @@ __device__ __forceinline__ void load_all(const SegArgs& s, const uint64_t (&pk)[
 }
 
 template <class C, int k>
-__device__ __forceinline__ void fold_from(const RawPack (&raw)[C::K], float (&acc)[kPack]) {
-    float v[kPack];
+__device__ __forceinline__ void fold_from(const RawPack (&raw)[C::K], float (&acc)[C::E]) {
+    float v[C::E];
     decode<C, k>(raw[k], v);
 #pragma unroll
-    for (int j = 0; j < kPack; ++j) acc[j] = step<C>(acc[j], v[j]);
+    for (int j = 0; j < C::E; ++j) acc[j] = step<C>(acc[j], v[j]);
     if constexpr (k + 1 < C::K) fold_from<C, k + 1>(raw, acc);
 }
 
 template <class C, int k>
-__device__ __forceinline__ void decode_all(const RawPack (&raw)[C::K], float (&v)[C::K][kPack]) {
+__device__ __forceinline__ void decode_all(const RawPack (&raw)[C::K], float (&v)[C::K][C::E]) {
     decode<C, k>(raw[k], v[k]);
     if constexpr (k + 1 < C::K) decode_all<C, k + 1>(raw, v);
 }
 
-// Reduce one packet's K operands to acc[8].
+// Reduce one packet's K operands to acc[E].
 template <class C>
-__device__ __forceinline__ void combine(const RawPack (&raw)[C::K], float (&acc)[kPack]) {
+__device__ __forceinline__ void combine(const RawPack (&raw)[C::K], float (&acc)[C::E]) {
     if constexpr (C::TOPO == MCCLX_TOPO_FOLD) {
         decode<C, 0>(raw[0], acc);
         if constexpr (C::K > 1) fold_from<C, 1>(raw, acc);
     } else {
         // allreduce_tree's reduce phase (AllreduceAlgos.cpp:100-114): at level
         // `mask` every surviving rank r (r % 2mask == 0) absorbs rank r+mask.
-        float v[C::K][kPack];
+        float v[C::K][C::E];
         decode_all<C, 0>(raw, v);
 #pragma unroll
         for (int mask = 1; mask < C::K; mask <<= 1)
 #pragma unroll
             for (int r = 0; r + mask < C::K; r += 2 * mask)
 #pragma unroll
-                for (int j = 0; j < kPack; ++j) v[r][j] = step<C>(v[r][j], v[r + mask][j]);
+                for (int j = 0; j < C::E; ++j) v[r][j] = step<C>(v[r][j], v[r + mask][j]);
 #pragma unroll
-        for (int j = 0; j < kPack; ++j) acc[j] = v[0][j];
+        for (int j = 0; j < C::E; ++j) acc[j] = v[0][j];
     }
 }
 
 template <class C>
-__device__ __forceinline__ void store_pack(const SegArgs& s, uint64_t pack, const float (&y)[kPack]) {
+__device__ __forceinline__ void store16(void* base, uint64_t pack, const float (&y)[C::E]) {
+    using V = Num<C::W>;
+    if constexpr (C::E == 8) {
+        u32x4 t;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t[j] = V::enc(y[2 * j]) | (V::enc(y[2 * j + 1]) << 16);
+        MCCLX_STG(gptr<u32x4_a2>(static_cast<uint16_t*>(base) + pack * C::E), t);
+    } else {
+        u32x2 t;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) t[j] = V::enc(y[2 * j]) | (V::enc(y[2 * j + 1]) << 16);
+        MCCLX_STG(gptr<u32x2_a2>(static_cast<uint16_t*>(base) + pack * C::E), t);
+    }
+}
+
+template <class C>
+__device__ __forceinline__ void store_pack(const SegArgs& s, uint64_t pack, const float (&y)[C::E]) {
     if constexpr (C::W == MCCLX_F32 || C::kOutF32) {
         if (s.out) {
-            u32x4 lo, hi;
+            u32x4 t;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                lo[j] = __float_as_uint(y[j]);
-                hi[j] = __float_as_uint(y[4 + j]);
-            }
-            MCCLX_GLOBAL Raw32* o = gptr<Raw32>(static_cast<float*>(s.out) + pack * kPack);
-            o->lo = lo;
-            o->hi = hi;
+            for (int j = 0; j < 4; ++j) t[j] = __float_as_uint(y[j]);
+            MCCLX_STG(gptr<u32x4_a4>(static_cast<float*>(s.out) + pack * C::E), t);
         }
     }
     if constexpr (C::W != MCCLX_F32) {
-        void* w = C::kOutF32 ? s.wire_out : (s.out ? s.out : s.wire_out);
-        if (w) {
-            u32x4 t;
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                t[j] = Num<C::W>::enc(y[2 * j]) | (Num<C::W>::enc(y[2 * j + 1]) << 16);
-            gptr<Raw16>(static_cast<uint16_t*>(w) + pack * kPack)->q = t;
-            if constexpr (!C::kOutF32)
-                if (s.out && s.wire_out)  // PURE with both outputs set
-                    gptr<Raw16>(static_cast<uint16_t*>(s.wire_out) + pack * kPack)->q = t;
+        if constexpr (C::kOutF32) {
+            if (s.wire_out) store16<C>(s.wire_out, pack, y);
+        } else {
+            if (s.out) store16<C>(s.out, pack, y);
+            if (s.wire_out) store16<C>(s.wire_out, pack, y);
         }
     }
 }
@@ -291,38 +340,73 @@ __device__ __forceinline__ void fold_packs(const SegArgs& s, const uint64_t (&pk
         RawPack col[C::K];
 #pragma unroll
         for (int k = 0; k < C::K; ++k) col[k] = raw[k][u];
-        float acc[kPack];
+        float acc[C::E];
         combine<C>(col, acc);
 #pragma unroll
-        for (int j = 0; j < kPack; ++j) acc[j] = finish<C>(acc[j], scale, has_scale);
+        for (int j = 0; j < C::E; ++j) acc[j] = finish<C>(acc[j], scale, has_scale);
         store_pack<C>(s, pk[u], acc);
     }
 }
 
-// The block's share of one segment: packets [first, P) in strides of `stride`
-// packets, plus the sub-packet tail when `do_tail`.
+// Elements in front of the packet grid: up to the 128-byte boundary of the
+// buffer the widest stores go to.
+template <class C>
+__device__ __forceinline__ uint32_t head_elems(const SegArgs& s) {
+#if MCCLX_TUNE_PEEL
+    const bool wide_out = (C::W == MCCLX_F32 || C::kOutF32) && s.out;
+    const uintptr_t a = reinterpret_cast<uintptr_t>(s.out ? s.out : s.wire_out);
+    const uint32_t es = wide_out ? 4u : 2u;
+    const uint32_t mis = (uint32_t)(a & 127u);
+    const uint64_t h = mis ? (128u - mis) / es : 0u;
+    return (uint32_t)(h < s.count ? h : s.count);
+#else
+    (void)s;
+    return 0;
+#endif
+}
+
+template <class C>
+__device__ __forceinline__ SegArgs shifted(const SegArgs& s, uint32_t head) {
+    SegArgs t;
+    const bool out_f32 = (C::W == MCCLX_F32 || C::kOutF32);
+    t.out = s.out ? static_cast<char*>(s.out) + (uint64_t)head * (out_f32 ? 4 : 2) : nullptr;
+    t.wire_out = s.wire_out ? static_cast<char*>(s.wire_out) + (uint64_t)head * 2 : nullptr;
+#pragma unroll
+    for (int k = 0; k < MCCLX_MAX_INPUTS; ++k)
+        t.in[k] = (k < C::K) ? static_cast<const char*>(s.in[k]) + (uint64_t)head * (C::in_is_f32(k) ? 4 : 2)
+                             : nullptr;
+    t.count = s.count - head;
+    return t;
+}
+
+// The block's share of one segment: after the head peel, packets [first, P) in
+// strides of `stride` packets; the block with `do_edges` also runs the head
+// and the sub-packet tail one element per lane.
 template <class C>
 __device__ __forceinline__ void fold_segment(const SegArgs& s, float scale, bool has_scale,
-                                             uint64_t first, uint64_t stride, bool do_tail) {
+                                             uint64_t first, uint64_t stride, bool do_edges) {
     constexpr int U = C::U;
-    const uint64_t P = s.count / kPack;
     const uint32_t tid = threadIdx.x;
+    const uint32_t head = head_elems<C>(s);  // < 64 <= kBlock
+    const SegArgs t = shifted<C>(s, head);
+    const uint64_t P = t.count / C::E;
     for (uint64_t base = first; base < P; base += stride) {
         if (base + (uint64_t)U * kBlock <= P) {
             uint64_t pk[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) pk[u] = base + (uint64_t)u * kBlock + tid;
-            fold_packs<C, U>(s, pk, scale, has_scale);
+            fold_packs<C, U>(t, pk, scale, has_scale);
         } else {
             for (uint64_t p = base + tid; p < P && p < base + (uint64_t)U * kBlock; p += kBlock) {
                 uint64_t one[1] = {p};
-                fold_packs<C, 1>(s, one, scale, has_scale);
+                fold_packs<C, 1>(t, one, scale, has_scale);
             }
         }
     }
-    if (do_tail) {
-        uint64_t i = P * kPack + tid;
-        if (i < s.count) fold_elem<C>(s, i, scale, has_scale);
+    if (do_edges) {
+        if (tid < head) fold_elem<C>(s, tid, scale, has_scale);
+        uint64_t i = P * C::E + tid;  // fewer than E <= 8 elements remain
+        if (i < t.count) fold_elem<C>(t, i, scale, has_scale);
     }
 }
 
@@ -375,7 +459,7 @@ __global__ void __launch_bounds__(kBlock) fold_table_kernel(TableArgs a) {
 
 template <class C>
 static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
-    const uint64_t span = (uint64_t)C::U * kBlock * kPack;  // elements per block iteration
+    const uint64_t span = (uint64_t)C::U * kBlock * C::E;  // elements per block iteration
     if (lp.table) {
         TableArgs a = *lp.table;
         uint32_t grid = (uint32_t)(a.total_items < lp.max_blocks ? a.total_items : lp.max_blocks);
@@ -395,23 +479,29 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
     return hipGetLastError();
 }
 
+static bool key_in_is_f32(const PlanKey& key, int k) {
+    return key.dtype == MCCLX_F32 || (key.io == MCCLX_IO_OWN_FIRST_F32 && k == 0) ||
+           (key.io == MCCLX_IO_OWN_LAST_F32 && k == key.k - 1);
+}
+static int key_pack_elems(const PlanKey& key) {
+    return (key.dtype == MCCLX_F32 || key.io != MCCLX_IO_PURE) ? 4 : 8;
+}
+
 uint32_t items_for(const PlanKey& k, uint64_t count) {
-    // must mirror Cfg::U for the plan; computed on the host for table building
-    uint64_t span = (uint64_t)plan_unroll(k) * kBlock * kPack;
+    // Mirrors Cfg::U / Cfg::E on the host, for table building.  The head peel
+    // only ever removes elements from the packet grid, so this is an upper
+    // bound; a tile past the end finds no packets and does nothing.
+    uint64_t span = (uint64_t)plan_unroll(k) * kBlock * key_pack_elems(k);
     uint64_t n = (count + span - 1) / span;
     return (uint32_t)(n ? n : (count ? 1 : 0));
 }
 
 int plan_unroll(const PlanKey& key) {
+    if (MCCLX_TUNE_U) return MCCLX_TUNE_U;
     if (key.topo == MCCLX_TOPO_BINOMIAL) return 1;
     int regs = 0;
-    for (int k = 0; k < key.k; ++k) {
-        bool f32 = key.dtype == MCCLX_F32 || (key.io == MCCLX_IO_OWN_FIRST_F32 && k == 0) ||
-                   (key.io == MCCLX_IO_OWN_LAST_F32 && k == key.k - 1);
-        regs += f32 ? 8 : 4;
-    }
-    int q = 64 / regs;
-    return q >= 4 ? 4 : q >= 2 ? 2 : 1;
+    for (int k = 0; k < key.k; ++k) regs += (key_in_is_f32(key, k) || key_pack_elems(key) == 8) ? 4 : 2;
+    return 32 / regs >= 2 ? 2 : 1;
 }
 
 #define MCCLX_K_CASES(W, IO, TOPO, OP, ACC)                                             \
@@ -451,6 +541,24 @@ int plan_unroll(const PlanKey& key) {
     }
 
 hipError_t launch_fold(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
+#ifdef MCCLX_TUNE_MINIMAL
+    // tuning builds: only the measured configurations, to keep compile times short
+    if (key.op == MCCLX_SUM && key.acc == MCCLX_ACC_STEP && key.topo == MCCLX_TOPO_FOLD) {
+        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_OWN_FIRST_F32 && key.k == 3)
+            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_OWN_FIRST_F32, 3, 0, 0, 0>>(st, lp);
+        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_OWN_FIRST_F32 && key.k == 1)
+            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_OWN_FIRST_F32, 1, 0, 0, 0>>(st, lp);
+        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_OWN_LAST_F32 && key.k == 4)
+            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_OWN_LAST_F32, 4, 0, 0, 0>>(st, lp);
+        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_PURE && key.k == 8)
+            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_PURE, 8, 0, 0, 0>>(st, lp);
+        if (key.dtype == MCCLX_F32 && key.k == 3)
+            return launch_cfg<Cfg<MCCLX_F32, MCCLX_IO_PURE, 3, 0, 0, 0>>(st, lp);
+        if (key.dtype == MCCLX_F32 && key.k == 2)
+            return launch_cfg<Cfg<MCCLX_F32, MCCLX_IO_PURE, 2, 0, 0, 0>>(st, lp);
+    }
+    return hipErrorInvalidValue;
+#else
     if (key.op != MCCLX_SUM) {
         if (key.io != MCCLX_IO_PURE || key.acc != MCCLX_ACC_STEP) return hipErrorInvalidValue;
         switch (key.dtype) {
@@ -485,6 +593,7 @@ hipError_t launch_fold(hipStream_t st, const PlanKey& key, const LaunchParams& l
         MCCLX_IO_CASES(MCCLX_ACC_F32)
     }
     return hipErrorInvalidValue;
+#endif
 }
 
 }  // namespace mcclx

@@ -86,6 +86,7 @@ struct mcclx_ctx {
     // re-recorded until 15 later waits have been issued
     hipEvent_t xev[16] = {};
     int xnext = 0;
+    hipStream_t upload_stream = nullptr;  // blocking table uploads while the queue is recording
 };
 
 namespace {
@@ -351,7 +352,12 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
         if (total == 0) return MCCLX_OK;
         void* dev = nullptr;
         HIP_TRY(hipMalloc(&dev, host.size()));
-        hipError_t ce = hipMemcpy(dev, host.data(), host.size(), hipMemcpyHostToDevice);
+        // not the legacy stream: that one may not be touched while another stream records
+        if (!ctx->upload_stream)
+            HIP_TRY(hipStreamCreateWithFlags(&ctx->upload_stream, hipStreamNonBlocking));
+        hipError_t ce = hipMemcpyAsync(dev, host.data(), host.size(), hipMemcpyHostToDevice,
+                                       ctx->upload_stream);
+        if (ce == hipSuccess) ce = hipStreamSynchronize(ctx->upload_stream);
         if (ce != hipSuccess) {
             (void)hipFree(dev);
             return fail(MCCLX_ERR_HIP, "table upload failed: %s", hipGetErrorString(ce));
@@ -479,6 +485,7 @@ int mcclx_destroy(mcclx_ctx* ctx) {
         if (sl.done) (void)hipEventDestroy(sl.done);
     }
     for (auto& kv : ctx->host_allocs) (void)hipHostFree(kv.first);
+    if (ctx->upload_stream) (void)hipStreamDestroy(ctx->upload_stream);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return MCCLX_OK;
