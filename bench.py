@@ -32,6 +32,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 CAL_BYTES = 64 << 20   # size of the calibration copy
+# HBM bytes one C2 fold launch moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by the
+# calibration copy (profiles/c2_fold_hbm_traffic_pmc.txt): 1.004 x the algorithmic bytes.
+C2_MEASURED_TRAFFIC_BYTES = 78_975_551
 
 
 def parse():
@@ -172,7 +175,7 @@ def main():
                                f"cold (rotating {args.sets} copies)",
                    "algorithmic_bytes_per_step": bytes_per_step, "parity_vs_oracle_bit_exact": parity},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": C2_MEASURED_TRAFFIC_BYTES,
                      "kernel": "fold_few_kernel<bf16, own-first fp32, k=3>", "kernel_us": round(kernel_us, 2)},
     }
     extra = {"warm_GBps": round(gbs(bytes_per_step, warm_dev / args.steps), 1),
