@@ -270,6 +270,12 @@ MCCLX_API int mcclx_reduce_scatter_replay(mcclx_ctx* ctx, int world, void* const
                                 const void* const* ins, int dtype, uint64_t chunk_numel, int op,
                                 int mode, int acc);
 
+/* The list form, reduce_scatter (ProcessGroupMCCL.cpp:392-464): shares[r*world + p]
+ * is rank p's contribution to rank r's output (chunk_numel elements each). */
+MCCLX_API int mcclx_reduce_scatter_shares(mcclx_ctx* ctx, int world, void* const* outs,
+                                const void* const* shares, int dtype, uint64_t chunk_numel,
+                                int op, int mode, int acc);
+
 /* _allgather_base (ProcessGroupMCCL.cpp:232-273): outs[r] = concat_p ins[p]. */
 MCCLX_API int mcclx_allgather_replay(mcclx_ctx* ctx, int world, void* const* outs, const void* const* ins,
                            uint64_t chunk_nbytes);

@@ -89,6 +89,7 @@ SIGNATURES = {
     "mcclx_replay_workspace_bytes": (_u64, [C.POINTER(Replay)]),
     "mcclx_allreduce_replay": (_i, [_vp, C.POINTER(Replay)]),
     "mcclx_reduce_scatter_replay": (_i, [_vp, _i, _pp, _pp, _i, _u64, _i, _i, _i]),
+    "mcclx_reduce_scatter_shares": (_i, [_vp, _i, _pp, _pp, _i, _u64, _i, _i, _i]),
     "mcclx_allgather_replay": (_i, [_vp, _i, _pp, _pp, _u64]),
 }
 

@@ -83,5 +83,61 @@ def build(force: bool = True, verbose: bool = False) -> str:
     return LIB_PATH
 
 
+BACKEND_DIR = os.path.join(CSRC, "backend")
+BACKEND_SOURCES = ["Progress.cpp", "LocalMesh.cpp", "WorkMCCL.cpp", "ProcessGroupMCCL.cpp", "bindings.cpp"]
+
+
+def backend_path() -> str:
+    import sysconfig
+    return os.path.join(HERE, "_C" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_backend(verbose: bool = False) -> str:
+    """Compile the c10d backend (host C++ against the installed torch) into
+    mccl_amd/_C*.so, linked against libmcclx.so next to it."""
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    if not os.path.exists(LIB_PATH):
+        build(force=True, verbose=verbose)
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    inc = ["-I" + p for p in ce.include_paths()] + ["-I" + sysconfig.get_paths()["include"],
+                                                     "-I/opt/rocm/include", "-I" + CSRC,
+                                                     "-I" + os.path.join(ROOT, "include")]
+    flags = ["-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wno-unused-parameter",
+             "-Wno-sign-compare", "-Wno-unknown-pragmas", "-pthread",
+             "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_C",
+             "-DTORCH_API_INCLUDE_EXTENSION_H",
+             "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI)]
+    procs, objs = [], []
+    for src in BACKEND_SOURCES:
+        obj = os.path.join(OBJ_DIR, "backend_" + os.path.splitext(src)[0] + ".o")
+        objs.append(obj)
+        cmd = ["g++"] + flags + inc + ["-c", os.path.join(BACKEND_DIR, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    for src, p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0:
+            raise RuntimeError(f"g++ failed on {src}:\n{out[-6000:]}")
+        if verbose and out.strip():
+            print(out[-3000:], flush=True)
+    out_path = backend_path()
+    tmp = out_path + ".tmp"
+    link = ["g++", "-shared", "-o", tmp] + objs + [
+        "-L" + HERE, "-lmcclx", "-L" + torch_lib, "-ltorch_python", "-ltorch", "-ltorch_cpu", "-ltorch_hip",
+        "-lc10", "-lc10_hip", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib, "-pthread"]
+    r = subprocess.run(link, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stdout}")
+    os.replace(tmp, out_path)
+    return out_path
+
+
 if __name__ == "__main__":
     print(build(force="--force" in sys.argv or needs_build(), verbose=True))
+    if "--backend" in sys.argv:
+        print(build_backend(verbose=True))

@@ -1,0 +1,84 @@
+#include "backend/LocalMesh.hpp"
+
+#include <atomic>
+#include <map>
+#include <unistd.h>
+
+#include "backend/Errors.hpp"
+
+namespace mccl {
+
+namespace {
+std::mutex g_registry_mu;
+std::map<std::string, std::weak_ptr<LocalMesh>> g_registry;
+std::atomic<uint64_t> g_next_id{1};
+}  // namespace
+
+std::string LocalMesh::fresh_key() {
+    return "pid" + std::to_string(::getpid()) + "-mesh" + std::to_string(g_next_id.fetch_add(1));
+}
+
+std::shared_ptr<LocalMesh> LocalMesh::create(const std::string& key, int world) {
+    auto mesh = std::make_shared<LocalMesh>(world);
+    std::lock_guard<std::mutex> lk(g_registry_mu);
+    g_registry[key] = mesh;
+    return mesh;
+}
+
+std::shared_ptr<LocalMesh> LocalMesh::find(const std::string& key) {
+    std::lock_guard<std::mutex> lk(g_registry_mu);
+    auto it = g_registry.find(key);
+    return it == g_registry.end() ? nullptr : it->second.lock();
+}
+
+void LocalMesh::forget(const std::string& key) {
+    std::lock_guard<std::mutex> lk(g_registry_mu);
+    auto it = g_registry.find(key);
+    if (it != g_registry.end() && it->second.expired()) g_registry.erase(it);
+}
+
+void LocalMesh::rendezvous(int rank, Contribution c, std::chrono::milliseconds timeout,
+                           const Leader& leader) {
+    std::unique_lock<std::mutex> lk(mu_);
+    MCCL_CHECK(rank >= 0 && rank < world_, "rank outside the mesh");
+    if (broken_) throw MCCLError("mesh is broken by an earlier timeout; the group cannot continue");
+    const uint64_t my_generation = generation_;
+    slots_[static_cast<size_t>(rank)] = std::move(c);
+    if (++arrived_ == world_) {
+        // Last arrival: every contribution is in.  Ranks must be inside the same collective.
+        std::exception_ptr err;
+        try {
+            for (int r = 1; r < world_; ++r)
+                MCCL_CHECK(slots_[static_cast<size_t>(r)].kind == slots_[0].kind,
+                           "ranks issued different collectives (rank 0 kind " +
+                               std::to_string(slots_[0].kind) + ", rank " + std::to_string(r) +
+                               " kind " + std::to_string(slots_[static_cast<size_t>(r)].kind) + ")");
+            leader(slots_);
+        } catch (...) {
+            err = std::current_exception();
+        }
+        last_error_ = err;
+        arrived_ = 0;
+        ++generation_;
+        lk.unlock();
+        cv_.notify_all();
+        if (err) std::rethrow_exception(err);
+        return;
+    }
+    auto released = [&] { return generation_ != my_generation || broken_; };
+    if (timeout.count() <= 0) {
+        cv_.wait(lk, released);
+    } else if (!cv_.wait_for(lk, timeout, released)) {
+        broken_ = true;
+        lk.unlock();
+        cv_.notify_all();
+        throw TimeoutError("rank " + std::to_string(rank) + ": peers did not reach the collective within " +
+                           std::to_string(timeout.count()) + " ms");
+    }
+    if (generation_ == my_generation && broken_)
+        throw TimeoutError("rank " + std::to_string(rank) + ": a peer timed out in this collective");
+    // generation advanced by exactly one: the error (if any) belongs to our collective
+    if (last_error_) std::rethrow_exception(last_error_);
+}
+
+}  // namespace mccl

@@ -1,0 +1,576 @@
+#include "backend/ProcessGroupMCCL.hpp"
+
+#include <c10/hip/HIPFunctions.h>
+#include <c10/hip/HIPStream.h>
+
+#include <condition_variable>
+#include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <map>
+#include <mutex>
+
+#include "backend/Errors.hpp"
+#include "backend/LocalMesh.hpp"
+#include "backend/Progress.hpp"
+#include "backend/WorkMCCL.hpp"
+
+namespace mccl {
+
+namespace {
+
+enum Kind { K_ALLREDUCE = 1, K_BROADCAST, K_ALLGATHER_BASE, K_ALLGATHER, K_REDUCE_SCATTER_BASE,
+            K_REDUCE_SCATTER, K_BARRIER };
+
+c10::intrusive_ptr<c10d::Work> make_completed(c10d::OpType op, std::vector<at::Tensor> outputs,
+                                              const char* title) {
+    auto w = c10::make_intrusive<WorkMCCL>(op, std::move(outputs), title);
+    w->finish();
+    return w;
+}
+
+c10::intrusive_ptr<c10d::Work> make_unimplemented(c10d::OpType op, std::vector<at::Tensor> outputs,
+                                                  const char* title) {
+    // the reference's make_unimplemented (ProcessGroupMCCL.cpp:38-43)
+    auto w = c10::make_intrusive<WorkMCCL>(op, std::move(outputs), title);
+    w->finishWithException(std::make_exception_ptr(MCCLError(
+        std::string(title) + ": not implemented (byte transport between processes is outside "
+                             "the single-GPU reduce path)")));
+    return w;
+}
+
+// check_mps_ (ProcessGroupMCCL.cpp:72-79) for ROCm tensors.
+void check_gpu_(const at::Tensor& t, const char* op) {
+    MCCL_CHECK(t.is_cuda(), std::string(op) + ": MCCL on MI355X is GPU-only; got " +
+                                std::string(c10::DeviceTypeName(t.device().type())) + " tensor");
+    MCCL_CHECK(t.is_contiguous(), std::string(op) + ": tensor must be contiguous");
+}
+
+// dtypes the reduce kernels cover (shaders.metal: f32 / f16 / bf16); -1 otherwise.
+int reduce_dtype(const at::Tensor& t) {
+    switch (t.scalar_type()) {
+        case at::kFloat: return MCCLX_F32;
+        case at::kHalf: return MCCLX_F16;
+        case at::kBFloat16: return MCCLX_BF16;
+        default: return -1;
+    }
+}
+
+int need_reduce_dtype(const at::Tensor& t, const char* op) {
+    int d = reduce_dtype(t);
+    // select_op_pipeline returns nil -> "No Metal pipeline for dtype" (MetalKernels.mm:634-635)
+    MCCL_CHECK(d >= 0, std::string(op) + ": No HIP kernel for dtype " + std::string(at::toString(t.scalar_type())));
+    return d;
+}
+
+int reduce_op_code(const c10d::ReduceOp& op) {
+    switch (static_cast<c10d::ReduceOp::RedOpType>(op)) {
+        case c10d::ReduceOp::SUM: return MCCLX_SUM;
+        case c10d::ReduceOp::AVG: return MCCLX_AVG;
+        case c10d::ReduceOp::PRODUCT: return MCCLX_PRODUCT;
+        case c10d::ReduceOp::MIN: return MCCLX_MIN;
+        case c10d::ReduceOp::MAX: return MCCLX_MAX;
+        default:
+            // MetalKernels.mm:546-548
+            throw MCCLError("Unsupported ReduceOp: " +
+                            std::to_string(static_cast<int>(static_cast<c10d::ReduceOp::RedOpType>(op))));
+    }
+}
+
+}  // namespace
+
+// One reduce queue and one grow-only scratch buffer per mesh (per group of
+// ranks sharing the GPU).  The scratch replaces the reference's per-call
+// at::empty recv buffers (ProcessGroupMCCL.cpp:152-162).
+struct ProcessGroupMCCL::Shared {
+    mcclx_ctx* ctx = nullptr;
+    at::Tensor scratch;
+    int device = 0;
+
+    ~Shared() {
+        if (ctx) mcclx_destroy(ctx);
+    }
+    void* workspace(uint64_t nbytes) {
+        if (nbytes == 0) return nullptr;
+        if (!scratch.defined() || static_cast<uint64_t>(scratch.numel()) < nbytes + 256) {
+            check_rc(mcclx_queue_drain(ctx));  // nothing may still read the old buffer
+            scratch = at::empty({static_cast<int64_t>(nbytes + 256)},
+                                at::TensorOptions().dtype(at::kByte).device(at::kCUDA, device));
+        }
+        auto p = reinterpret_cast<uintptr_t>(scratch.data_ptr());
+        return reinterpret_cast<void*>((p + 255) / 256 * 256);
+    }
+};
+
+namespace {
+std::mutex g_shared_mu;
+std::map<std::string, std::weak_ptr<void>> g_shared;  // mesh key -> Shared (type-erased)
+}  // namespace
+
+ProcessGroupMCCL::ProcessGroupMCCL(c10::intrusive_ptr<c10d::Store> store, int rank, int size, Options opts)
+    : c10d::Backend(rank, size), store_(std::move(store)), opts_(opts) {
+    MCCL_CHECK(rank >= 0 && rank < size, "rank/size invalid");
+    try {
+        device_ = static_cast<int>(c10::hip::current_device());
+    } catch (const std::exception& e) {
+        // the reference fails in metal_kernels_init() when there is no Metal device
+        throw MCCLError(std::string("no usable GPU for the mccl backend: ") + e.what());
+    }
+    if (size == 1) {
+        // metal_kernels_init() (ProcessGroupMCCL.cpp:93): fails loudly without a GPU
+        shared_ = std::make_shared<Shared>();
+        shared_->device = device_;
+        check_rc(mcclx_init(device_, &shared_->ctx));
+        ctx_ = shared_->ctx;
+        return;
+    }
+    // Rendezvous through the store (the reference exchanges TCP endpoints here,
+    // runtime/Rendezvous.cpp:23-79): rank 0 publishes the key of the in-process mesh.
+    const std::string store_key = "mccl/local_mesh";
+    if (rank == 0) {
+        mesh_key_ = LocalMesh::fresh_key();
+        mesh_ = LocalMesh::create(mesh_key_, size);
+        auto sh = std::make_shared<Shared>();
+        sh->device = device_;
+        check_rc(mcclx_init(device_, &sh->ctx));
+        {
+            std::lock_guard<std::mutex> lk(g_shared_mu);
+            g_shared[mesh_key_] = sh;
+        }
+        shared_ = sh;
+        store_->set(store_key, std::vector<uint8_t>(mesh_key_.begin(), mesh_key_.end()));
+    } else {
+        auto raw = store_->get(store_key);  // blocks until rank 0 has set it (store timeout applies)
+        mesh_key_.assign(raw.begin(), raw.end());
+        mesh_ = LocalMesh::find(mesh_key_);
+        MCCL_CHECK(mesh_ != nullptr,
+                   "rank 0 of this group is not in this process: this build runs all ranks of a "
+                   "group in one process on one GPU");
+        MCCL_CHECK(mesh_->world() == size, "mesh size differs from group size");
+        std::lock_guard<std::mutex> lk(g_shared_mu);
+        shared_ = std::static_pointer_cast<Shared>(g_shared[mesh_key_].lock());
+        MCCL_CHECK(shared_ != nullptr, "mesh context already destroyed");
+    }
+    ctx_ = shared_->ctx;
+    engine_ = std::make_unique<Progress>();
+}
+
+ProcessGroupMCCL::~ProcessGroupMCCL() {
+    if (engine_) engine_->shutdown();
+    mesh_.reset();
+    shared_.reset();
+    if (!mesh_key_.empty()) LocalMesh::forget(mesh_key_);
+}
+
+void* ProcessGroupMCCL::my_stream() const {
+    return static_cast<void*>(c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(device_)).stream());
+}
+
+void ProcessGroupMCCL::meet(Contribution c, const LocalMesh::Leader& leader) {
+    mesh_->rendezvous(getRank(), std::move(c), opts_.timeout, leader);
+}
+
+// The allreduce runs on the caller's thread while every other collective runs
+// on the engine thread (as in the reference); a rank must not enter the
+// allreduce's meeting point while its own engine still owes an earlier
+// collective, or the ranks would meet in different collectives.
+void ProcessGroupMCCL::flush_engine_() {
+    if (!engine_) return;
+    std::mutex mu;
+    std::condition_variable cv;
+    bool done = false;
+    engine_->submit([&] {
+        std::lock_guard<std::mutex> lk(mu);
+        done = true;
+        cv.notify_all();
+    });
+    std::unique_lock<std::mutex> lk(mu);
+    cv.wait(lk, [&] { return done; });
+}
+
+namespace {
+
+// Asynchronous shell of the reference (async_submit_, ProcessGroupMCCL.cpp:45-70):
+// the issuing thread orders the reduce queue after its own stream (the
+// reference records an event on torch's stream there), the engine thread runs
+// the body and completes the Work; the sync callback drains the queue first.
+c10::intrusive_ptr<c10d::Work> async_submit_(Progress& engine, mcclx_ctx* ctx, void* issuing_stream,
+                                             c10d::OpType op, std::vector<at::Tensor> outputs,
+                                             const char* title, std::function<void()> body) {
+    auto work = c10::make_intrusive<WorkMCCL>(op, std::move(outputs), title);
+    try {
+        check_rc(mcclx_queue_wait_stream(ctx, issuing_stream));
+    } catch (...) {
+        work->finishWithException(std::current_exception());
+        return work;
+    }
+    work->setSyncCallback([ctx] { check_rc(mcclx_queue_drain(ctx)); });
+    engine.submit([work, body = std::move(body)]() {
+        try {
+            body();
+            work->finish();
+        } catch (...) {
+            work->finishWithException(std::current_exception());
+        }
+    });
+    return work;
+}
+
+bool env_wire_bf16() {
+    const char* w = std::getenv("MCCL_WIRE_DTYPE");  // re-read on every call (ProcessGroupMCCL.cpp:117-120)
+    return w && std::strcmp(w, "bf16") == 0;
+}
+
+int64_t env_tree_below() {
+    const char* e = std::getenv("MCCL_TREE_BELOW");  // :138-139
+    return e ? static_cast<int64_t>(std::strtoull(e, nullptr, 10)) : -1;
+}
+
+}  // namespace
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tensor>& tensors,
+                                                           const c10d::AllreduceOptions& opts) {
+    if (getSize() == 1) return make_completed(c10d::OpType::ALLREDUCE, tensors, "mccl:allreduce");
+    MCCL_CHECK(!tensors.empty(), "allreduce: empty tensor list");
+    const int op = reduce_op_code(opts.reduceOp);
+    const int world = getSize();
+    const bool wire = env_wire_bf16();
+    const char* env_alg = std::getenv("MCCL_ALLREDUCE_ALGO");
+    const int64_t tree_below = env_tree_below();
+
+    Contribution c;
+    c.kind = K_ALLREDUCE;
+    c.op = op;
+    c.wire_bf16 = wire ? 1 : 0;
+    c.stream = my_stream();
+    for (auto& t : tensors) {
+        check_gpu_(t, "allreduce");
+        const int dt = need_reduce_dtype(t, "allreduce");
+        MCCL_CHECK(t.numel() > 0, "MCCL does not accept empty tensors");  // TensorChecks.hpp:31-34
+        const bool use_wire = wire && dt == MCCLX_F32;  // :131
+        const uint64_t bytes = static_cast<uint64_t>(t.numel()) * (use_wire ? 2u : t.element_size());
+        c.dst.push_back(t.data_ptr());
+        c.numel.push_back(static_cast<uint64_t>(t.numel()));
+        c.dtype.push_back(dt);
+        c.algo.push_back(mcclx_select_algo(env_alg, tree_below, bytes, t.numel(), world));  // :134-145
+    }
+    last_algo_ = c.algo.back();
+    flush_engine_();
+
+    auto shared = shared_;
+    // The allreduce is synchronous, as in the reference (ProcessGroupMCCL.cpp:170-185):
+    // when it returns, every rank's tensor holds the result and the queue is drained.
+    meet(std::move(c), [shared, world](const std::vector<Contribution>& all) {
+        mcclx_ctx* ctx = shared->ctx;
+        const size_t nt = all[0].dst.size();
+        for (int r = 0; r < world; ++r) {
+            MCCL_CHECK(all[r].dst.size() == nt, "allreduce: ranks passed different numbers of tensors");
+            MCCL_CHECK(all[r].op == all[0].op && all[r].wire_bf16 == all[0].wire_bf16,
+                       "allreduce: ranks disagree on the reduce op or MCCL_WIRE_DTYPE");
+            check_rc(mcclx_queue_wait_stream(ctx, all[r].stream));  // mps_stream_sync, :172
+        }
+        for (size_t i = 0; i < nt; ++i) {
+            std::vector<void*> ptrs(static_cast<size_t>(world));
+            for (int r = 0; r < world; ++r) {
+                MCCL_CHECK(all[r].numel[i] == all[0].numel[i] && all[r].dtype[i] == all[0].dtype[i],
+                           "allreduce: ranks passed tensors of different size or dtype");
+                MCCL_CHECK(all[r].algo[i] == all[0].algo[i],
+                           "allreduce: ranks resolved different algorithms (MCCL_ALLREDUCE_ALGO / MCCL_TREE_BELOW differ)");
+                ptrs[static_cast<size_t>(r)] = all[r].dst[i];
+            }
+            mcclx_replay rp;
+            std::memset(&rp, 0, sizeof rp);
+            rp.world = world;
+            rp.algo = all[0].algo[i];
+            rp.op = all[0].op;
+            rp.dtype = all[0].dtype[i];
+            rp.wire_bf16 = all[0].wire_bf16;
+            rp.mode = MCCLX_REPLAY_FUSED;
+            rp.acc = MCCLX_ACC_STEP;
+            rp.numel = all[0].numel[i];
+            rp.tensors = ptrs.data();
+            // size for the stepwise fallback too (binary-only ops, wide worlds)
+            mcclx_replay st = rp;
+            st.mode = MCCLX_REPLAY_STEPWISE;
+            uint64_t need = std::max(mcclx_replay_workspace_bytes(&rp), mcclx_replay_workspace_bytes(&st));
+            rp.workspace = shared->workspace(need);
+            rp.workspace_bytes = need;
+            check_rc(mcclx_allreduce_replay(ctx, &rp));
+        }
+        check_rc(mcclx_queue_drain(ctx));  // mccl_queue_drain, :178
+    });
+    return make_completed(c10d::OpType::ALLREDUCE, tensors, "mccl:allreduce");
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::broadcast(std::vector<at::Tensor>& tensors,
+                                                           const c10d::BroadcastOptions& opts) {
+    if (getSize() == 1) return make_completed(c10d::OpType::BROADCAST, tensors, "mccl:broadcast");
+    MCCL_CHECK(!tensors.empty(), "broadcast: empty tensor list");
+    auto tensors_copy = tensors;
+    const int root = static_cast<int>(opts.rootRank);
+    const int world = getSize();
+    auto shared = shared_;
+    void* stream = my_stream();
+    return async_submit_(*engine_, ctx_, stream, c10d::OpType::BROADCAST, tensors, "mccl:broadcast",
+                         [this, shared, tensors_copy, root, world, stream]() mutable {
+        Contribution c;
+        c.kind = K_BROADCAST;
+        c.root = root;
+        c.stream = stream;
+        for (auto& t : tensors_copy) {
+            check_gpu_(t, "broadcast");
+            c.dst.push_back(t.data_ptr());
+            c.nbytes.push_back(static_cast<uint64_t>(t.nbytes()));
+        }
+        meet(std::move(c), [shared, world](const std::vector<Contribution>& all) {
+            const int root = all[0].root;
+            MCCL_CHECK(root >= 0 && root < world, "broadcast: root outside the group");
+            for (int r = 0; r < world; ++r) {
+                MCCL_CHECK(all[r].root == root && all[r].dst.size() == all[0].dst.size(),
+                           "broadcast: ranks disagree on root or tensor count");
+                check_rc(mcclx_queue_wait_stream(shared->ctx, all[r].stream));
+            }
+            for (size_t i = 0; i < all[0].dst.size(); ++i)
+                for (int r = 0; r < world; ++r) {
+                    if (r == root) continue;
+                    MCCL_CHECK(all[r].nbytes[i] == all[root].nbytes[i], "broadcast: size mismatch");
+                    check_rc(mcclx_copy(shared->ctx, all[r].dst[i], all[root].dst[i], all[root].nbytes[i]));
+                }
+        });
+    });
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::_allgather_base(at::Tensor& output_tensor,
+                                                                 at::Tensor& input_tensor,
+                                                                 const c10d::AllgatherOptions&) {
+    if (getSize() == 1) {
+        output_tensor.copy_(input_tensor);
+        return make_completed(c10d::OpType::_ALLGATHER_BASE, {output_tensor}, "mccl:_allgather_base");
+    }
+    at::Tensor out = output_tensor, in = input_tensor;
+    const int world = getSize();
+    auto shared = shared_;
+    void* stream = my_stream();
+    return async_submit_(*engine_, ctx_, stream, c10d::OpType::_ALLGATHER_BASE, {output_tensor},
+                         "mccl:_allgather_base", [this, shared, out, in, world, stream]() mutable {
+        check_gpu_(in, "_allgather_base");
+        check_gpu_(out, "_allgather_base");
+        const uint64_t chunk = static_cast<uint64_t>(in.nbytes());
+        MCCL_CHECK(static_cast<uint64_t>(out.nbytes()) == chunk * static_cast<uint64_t>(world),
+                   "_allgather_base: output size != input * world");
+        Contribution c;
+        c.kind = K_ALLGATHER_BASE;
+        c.stream = stream;
+        c.dst = {out.data_ptr()};
+        c.src = {in.data_ptr()};
+        c.nbytes = {chunk};
+        meet(std::move(c), [shared, world](const std::vector<Contribution>& all) {
+            std::vector<void*> outs(static_cast<size_t>(world));
+            std::vector<const void*> ins(static_cast<size_t>(world));
+            for (int r = 0; r < world; ++r) {
+                MCCL_CHECK(all[r].nbytes[0] == all[0].nbytes[0], "_allgather_base: ranks pass different sizes");
+                outs[static_cast<size_t>(r)] = all[r].dst[0];
+                ins[static_cast<size_t>(r)] = all[r].src[0];
+                check_rc(mcclx_queue_wait_stream(shared->ctx, all[r].stream));
+            }
+            check_rc(mcclx_allgather_replay(shared->ctx, world, outs.data(), ins.data(), all[0].nbytes[0]));
+        });
+    });
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allgather(
+    std::vector<std::vector<at::Tensor>>& output_tensors, std::vector<at::Tensor>& input_tensors,
+    const c10d::AllgatherOptions&) {
+    if (getSize() == 1) {
+        MCCL_CHECK(!output_tensors.empty() && !output_tensors[0].empty(), "allgather output empty");
+        output_tensors[0][0].copy_(input_tensors[0]);
+        return make_completed(c10d::OpType::ALLGATHER, output_tensors[0], "mccl:allgather");
+    }
+    auto outs_copy = output_tensors;
+    auto ins_copy = input_tensors;
+    const int world = getSize();
+    auto shared = shared_;
+    void* stream = my_stream();
+    return async_submit_(*engine_, ctx_, stream, c10d::OpType::ALLGATHER, input_tensors, "mccl:allgather",
+                         [this, shared, outs_copy, ins_copy, world, stream]() mutable {
+        MCCL_CHECK(ins_copy.size() == outs_copy.size(), "allgather: input/output count mismatch");
+        Contribution c;
+        c.kind = K_ALLGATHER;
+        c.stream = stream;
+        for (size_t i = 0; i < ins_copy.size(); ++i) {
+            MCCL_CHECK(static_cast<int>(outs_copy[i].size()) == world, "allgather: output list size != world");
+            check_gpu_(ins_copy[i], "allgather");
+            c.src.push_back(ins_copy[i].data_ptr());
+            c.nbytes.push_back(static_cast<uint64_t>(ins_copy[i].nbytes()));
+            for (auto& o : outs_copy[i]) {
+                check_gpu_(o, "allgather");
+                MCCL_CHECK(o.nbytes() == ins_copy[i].nbytes(), "allgather: output size != input size");
+                c.dst.push_back(o.data_ptr());
+            }
+        }
+        meet(std::move(c), [shared, world](const std::vector<Contribution>& all) {
+            for (int r = 0; r < world; ++r) check_rc(mcclx_queue_wait_stream(shared->ctx, all[r].stream));
+            const size_t nt = all[0].src.size();
+            for (size_t i = 0; i < nt; ++i)
+                for (int r = 0; r < world; ++r) {
+                    MCCL_CHECK(all[r].src.size() == nt && all[r].nbytes[i] == all[0].nbytes[i],
+                               "allgather: ranks pass different tensors");
+                    for (int p = 0; p < world; ++p)
+                        check_rc(mcclx_copy(shared->ctx, all[r].dst[i * static_cast<size_t>(world) + p],
+                                            all[p].src[i], all[0].nbytes[i]));
+                }
+        });
+    });
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::_reduce_scatter_base(at::Tensor& output_tensor,
+                                                                      at::Tensor& input_tensor,
+                                                                      const c10d::ReduceScatterOptions& opts) {
+    if (getSize() == 1) {
+        output_tensor.copy_(input_tensor);
+        return make_completed(c10d::OpType::_REDUCE_SCATTER_BASE, {output_tensor}, "mccl:_reduce_scatter_base");
+    }
+    const int op = reduce_op_code(opts.reduceOp);
+    at::Tensor out = output_tensor, in = input_tensor;
+    const int world = getSize();
+    auto shared = shared_;
+    void* stream = my_stream();
+    return async_submit_(*engine_, ctx_, stream, c10d::OpType::_REDUCE_SCATTER_BASE, {output_tensor},
+                         "mccl:_reduce_scatter_base", [this, shared, out, in, op, world, stream]() mutable {
+        check_gpu_(in, "_reduce_scatter_base");
+        check_gpu_(out, "_reduce_scatter_base");
+        MCCL_CHECK(static_cast<uint64_t>(in.nbytes()) == static_cast<uint64_t>(out.nbytes()) * world,
+                   "_reduce_scatter_base: input size != output * world");
+        Contribution c;
+        c.kind = K_REDUCE_SCATTER_BASE;
+        c.op = op;
+        c.stream = stream;
+        c.dst = {out.data_ptr()};
+        c.src = {in.data_ptr()};
+        c.numel = {static_cast<uint64_t>(out.numel())};
+        c.dtype = {need_reduce_dtype(out, "_reduce_scatter_base")};
+        MCCL_CHECK(in.scalar_type() == out.scalar_type(), "_reduce_scatter_base: dtype mismatch");
+        meet(std::move(c), [shared, world](const std::vector<Contribution>& all) {
+            std::vector<void*> outs(static_cast<size_t>(world));
+            std::vector<const void*> ins(static_cast<size_t>(world));
+            for (int r = 0; r < world; ++r) {
+                MCCL_CHECK(all[r].numel[0] == all[0].numel[0] && all[r].dtype[0] == all[0].dtype[0] &&
+                               all[r].op == all[0].op,
+                           "_reduce_scatter_base: ranks disagree on size, dtype or op");
+                outs[static_cast<size_t>(r)] = all[r].dst[0];
+                ins[static_cast<size_t>(r)] = all[r].src[0];
+                check_rc(mcclx_queue_wait_stream(shared->ctx, all[r].stream));
+            }
+            // one launch for the whole group (the reference batches its N-1 binary
+            // launches per rank into one command buffer, :378-387)
+            check_rc(mcclx_batch_begin(shared->ctx, "mccl:_reduce_scatter_base"));
+            int rc = mcclx_reduce_scatter_replay(shared->ctx, world, outs.data(), ins.data(), all[0].dtype[0],
+                                                 all[0].numel[0], all[0].op, MCCLX_REPLAY_FUSED, MCCLX_ACC_STEP);
+            mcclx_batch_end(shared->ctx);
+            check_rc(rc);
+        });
+    });
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::reduce_scatter(
+    std::vector<at::Tensor>& output_tensors, std::vector<std::vector<at::Tensor>>& input_tensors,
+    const c10d::ReduceScatterOptions& opts) {
+    if (getSize() == 1) {
+        MCCL_CHECK(!input_tensors.empty() && !input_tensors[0].empty(), "reduce_scatter input empty");
+        output_tensors[0].copy_(input_tensors[0][0]);
+        return make_completed(c10d::OpType::REDUCE_SCATTER, output_tensors, "mccl:reduce_scatter");
+    }
+    const int op = reduce_op_code(opts.reduceOp);
+    auto outs_copy = output_tensors;
+    auto ins_copy = input_tensors;
+    const int world = getSize();
+    auto shared = shared_;
+    void* stream = my_stream();
+    return async_submit_(*engine_, ctx_, stream, c10d::OpType::REDUCE_SCATTER, output_tensors,
+                         "mccl:reduce_scatter", [this, shared, outs_copy, ins_copy, op, world, stream]() mutable {
+        MCCL_CHECK(outs_copy.size() == ins_copy.size(), "reduce_scatter: count mismatch");
+        Contribution c;
+        c.kind = K_REDUCE_SCATTER;
+        c.op = op;
+        c.stream = stream;
+        for (size_t i = 0; i < outs_copy.size(); ++i) {
+            auto& out = outs_copy[i];
+            auto& ins = ins_copy[i];
+            MCCL_CHECK(static_cast<int>(ins.size()) == world, "reduce_scatter: input list size != world");
+            check_gpu_(out, "reduce_scatter");
+            c.dst.push_back(out.data_ptr());
+            c.numel.push_back(static_cast<uint64_t>(out.numel()));
+            c.dtype.push_back(need_reduce_dtype(out, "reduce_scatter"));
+            for (auto& t : ins) {
+                check_gpu_(t, "reduce_scatter");
+                MCCL_CHECK(t.nbytes() == out.nbytes() && t.scalar_type() == out.scalar_type(),
+                           "reduce_scatter: output size != input chunk size");
+                c.src.push_back(t.data_ptr());
+            }
+        }
+        meet(std::move(c), [shared, world](const std::vector<Contribution>& all) {
+            for (int r = 0; r < world; ++r) check_rc(mcclx_queue_wait_stream(shared->ctx, all[r].stream));
+            const size_t nt = all[0].dst.size();
+            const size_t W = static_cast<size_t>(world);
+            for (size_t i = 0; i < nt; ++i) {
+                std::vector<void*> outs(W);
+                std::vector<const void*> shares(W * W);
+                for (size_t r = 0; r < W; ++r) {
+                    MCCL_CHECK(all[r].dst.size() == nt && all[r].numel[i] == all[0].numel[i] &&
+                                   all[r].dtype[i] == all[0].dtype[i] && all[r].op == all[0].op,
+                               "reduce_scatter: ranks disagree on size, dtype or op");
+                    outs[r] = all[r].dst[i];
+                    // rank p's list entry r is its contribution to rank r's output
+                    for (size_t p = 0; p < W; ++p) shares[r * W + p] = all[p].src[i * W + r];
+                }
+                check_rc(mcclx_reduce_scatter_shares(shared->ctx, world, outs.data(), shares.data(),
+                                                     all[0].dtype[i], all[0].numel[i], all[0].op,
+                                                     MCCLX_REPLAY_FUSED, MCCLX_ACC_STEP));
+            }
+        });
+    });
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::barrier(const c10d::BarrierOptions&) {
+    if (getSize() == 1) return make_completed(c10d::OpType::BARRIER, {}, "mccl:barrier");
+    auto shared = shared_;
+    void* stream = my_stream();
+    return async_submit_(*engine_, ctx_, stream, c10d::OpType::BARRIER, {}, "mccl:barrier",
+                         [this, stream]() {
+        Contribution c;
+        c.kind = K_BARRIER;
+        c.stream = stream;
+        meet(std::move(c), [](const std::vector<Contribution>&) {});
+    });
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::alltoall_base(at::Tensor& output_tensor, at::Tensor& input_tensor,
+                                                               std::vector<int64_t>&, std::vector<int64_t>&,
+                                                               const c10d::AllToAllOptions&) {
+    if (getSize() == 1) {
+        output_tensor.copy_(input_tensor);
+        return make_completed(c10d::OpType::ALLTOALL_BASE, {output_tensor}, "mccl:alltoall_base");
+    }
+    return make_unimplemented(c10d::OpType::ALLTOALL_BASE, {output_tensor}, "mccl:alltoall_base");
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::alltoall(std::vector<at::Tensor>& output_tensors,
+                                                          std::vector<at::Tensor>& input_tensors,
+                                                          const c10d::AllToAllOptions&) {
+    if (getSize() == 1) {
+        MCCL_CHECK(!output_tensors.empty() && !input_tensors.empty(), "alltoall tensors empty");
+        output_tensors[0].copy_(input_tensors[0]);
+        return make_completed(c10d::OpType::ALLTOALL, output_tensors, "mccl:alltoall");
+    }
+    return make_unimplemented(c10d::OpType::ALLTOALL, output_tensors, "mccl:alltoall");
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::send(std::vector<at::Tensor>& tensors, int, int) {
+    return make_unimplemented(c10d::OpType::SEND, tensors, "mccl:send");
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::recv(std::vector<at::Tensor>& tensors, int, int) {
+    return make_unimplemented(c10d::OpType::RECV, tensors, "mccl:recv");
+}
+
+}  // namespace mccl

@@ -1,0 +1,53 @@
+#include "backend/Progress.hpp"
+
+#include <utility>
+
+namespace mccl {
+
+Progress::Progress() { thread_ = std::thread([this] { worker(); }); }
+
+Progress::~Progress() { shutdown(); }
+
+void Progress::submit(Task task) {
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        if (closing_) return;
+        queue_.push_back(std::move(task));
+    }
+    wake_.notify_one();
+}
+
+void Progress::shutdown() {
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        if (closing_ && !thread_.joinable()) return;
+        closing_ = true;
+    }
+    wake_.notify_all();
+    if (thread_.joinable()) thread_.join();
+}
+
+size_t Progress::completed() const {
+    std::lock_guard<std::mutex> lk(mu_);
+    return completed_;
+}
+
+void Progress::worker() {
+    std::unique_lock<std::mutex> lk(mu_);
+    for (;;) {
+        wake_.wait(lk, [this] { return closing_ || !queue_.empty(); });
+        if (queue_.empty()) return;  // closing and drained
+        Task task = std::move(queue_.front());
+        queue_.pop_front();
+        lk.unlock();
+        try {
+            task();
+        } catch (...) {
+            // the task reports its own failure through its Work object
+        }
+        lk.lock();
+        ++completed_;
+    }
+}
+
+}  // namespace mccl

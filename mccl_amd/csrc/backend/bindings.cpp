@@ -1,0 +1,164 @@
+// bindings.cpp -- the `mccl_amd._C` extension module.
+//
+// Exposes the factory torch.distributed needs, mirroring the reference's
+// csrc/backend/Registration.cpp:22-39 (`_create_process_group_mccl(store, rank,
+// size, timeout)`), plus small host-only hooks the CPU tests drive (the FIFO
+// engine, the Work object, the in-process mesh).
+#include <torch/extension.h>
+
+#include <pybind11/chrono.h>
+#include <pybind11/functional.h>
+#include <pybind11/stl.h>
+
+#include <torch/csrc/distributed/c10d/Backend.hpp>
+#include <torch/csrc/distributed/c10d/Store.hpp>
+
+#include <atomic>
+#include <chrono>
+#include <thread>
+
+#include "backend/Errors.hpp"
+#include "backend/LocalMesh.hpp"
+#include "backend/ProcessGroupMCCL.hpp"
+#include "backend/Progress.hpp"
+#include "backend/WorkMCCL.hpp"
+
+namespace py = pybind11;
+
+namespace {
+
+// Submits n tasks; task i throws when bit i of throw_mask is set (i < 64).
+// Returns the order in which the non-throwing tasks ran.
+std::vector<int> progress_order(int n, uint64_t throw_mask, bool use_destructor) {
+    std::vector<int> order;
+    std::mutex mu;
+    {
+        mccl::Progress p;
+        for (int i = 0; i < n; ++i) {
+            const bool thr = i < 64 && ((throw_mask >> i) & 1u);
+            p.submit([i, thr, &order, &mu] {
+                if (thr) throw std::runtime_error("boom");
+                std::lock_guard<std::mutex> lk(mu);
+                order.push_back(i);
+            });
+        }
+        if (!use_destructor) {
+            p.shutdown();
+            p.shutdown();  // idempotent
+        }
+    }
+    return order;
+}
+
+// Microseconds a submit() takes while the worker is busy with a 50 ms task.
+long progress_submit_latency_us() {
+    mccl::Progress p;
+    p.submit([] { std::this_thread::sleep_for(std::chrono::milliseconds(50)); });
+    auto t0 = std::chrono::steady_clock::now();
+    p.submit([] {});
+    auto t1 = std::chrono::steady_clock::now();
+    p.shutdown();
+    return static_cast<long>(std::chrono::duration_cast<std::chrono::microseconds>(t1 - t0).count());
+}
+
+// Exercises WorkMCCL without any device: returns (completed, success, message).
+std::tuple<bool, bool, std::string> work_probe(const std::string& mode, int wait_ms) {
+    auto w = c10::make_intrusive<mccl::WorkMCCL>(c10d::OpType::ALLREDUCE, std::vector<at::Tensor>{}, "mccl:test");
+    std::string msg;
+    if (mode == "finish") {
+        w->finish();
+        w->finish();
+    } else if (mode == "fail") {
+        w->finishWithException(std::make_exception_ptr(mccl::MCCLError("engine task failed")));
+        w->finish();  // too late: the first completion stands
+    } else if (mode == "sync_cb_throws") {
+        w->setSyncCallback([] { throw mccl::MCCLError("drain failed"); });
+        w->finish();
+    } else if (mode == "late") {
+        std::thread([w] {
+            std::this_thread::sleep_for(std::chrono::milliseconds(30));
+            w->finish();
+        }).detach();
+    }
+    bool ok = false;
+    try {
+        ok = w->wait(std::chrono::milliseconds(wait_ms));
+        if (!ok) msg = "timeout";
+    } catch (const std::exception& e) {
+        msg = e.what();
+    }
+    if (mode == "late") w->wait();
+    bool future_err = w->getFuture()->completed() && w->getFuture()->hasError();
+    return {w->isCompleted(), w->isSuccess() && !future_err, msg};
+}
+
+// N threads meet `rounds` times in a LocalMesh; rank `absent` (if >= 0) never
+// shows up, rank `thrower` makes the leader throw.  Returns per-rank messages.
+std::vector<std::string> mesh_probe(int world, int rounds, int absent, int timeout_ms, bool leader_throws) {
+    auto mesh = mccl::LocalMesh::create(mccl::LocalMesh::fresh_key(), world);
+    std::vector<std::string> out(static_cast<size_t>(world));
+    std::vector<std::thread> ts;
+    std::atomic<int> leader_runs{0};
+    for (int r = 0; r < world; ++r) {
+        if (r == absent) {
+            out[static_cast<size_t>(r)] = "absent";
+            continue;
+        }
+        ts.emplace_back([&, r] {
+            try {
+                for (int i = 0; i < rounds; ++i) {
+                    mccl::Contribution c;
+                    c.kind = 100 + i;
+                    c.numel = {static_cast<uint64_t>(r)};
+                    mesh->rendezvous(r, c, std::chrono::milliseconds(timeout_ms),
+                                     [&](const std::vector<mccl::Contribution>& all) {
+                                         for (int q = 0; q < world; ++q)
+                                             if (all[static_cast<size_t>(q)].numel[0] != static_cast<uint64_t>(q))
+                                                 throw mccl::MCCLError("slot mix-up");
+                                         ++leader_runs;
+                                         if (leader_throws) throw mccl::MCCLError("leader failed");
+                                     });
+                }
+                out[static_cast<size_t>(r)] = "ok:" + std::to_string(leader_runs.load());
+            } catch (const std::exception& e) {
+                out[static_cast<size_t>(r)] = e.what();
+            }
+        });
+    }
+    for (auto& t : ts) t.join();
+    return out;
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    m.doc() = "mccl_amd native backend: c10d ProcessGroup over libmcclx";
+    py::register_exception<mccl::MCCLError>(m, "MCCLError", PyExc_RuntimeError);
+
+    m.def("_create_process_group_mccl",
+          [](const c10::intrusive_ptr<c10d::Store>& store, int rank, int size,
+             std::chrono::milliseconds timeout) -> c10::intrusive_ptr<c10d::Backend> {
+              mccl::ProcessGroupMCCL::Options opts;
+              opts.timeout = timeout;
+              return c10::make_intrusive<mccl::ProcessGroupMCCL>(store, rank, size, opts);
+          },
+          py::arg("store"), py::arg("rank"), py::arg("size"),
+          py::arg("timeout") = std::chrono::milliseconds(30 * 60 * 1000),
+          py::call_guard<py::gil_scoped_release>(),
+          "Factory used by torch.distributed.Backend.register_backend('mccl').");
+
+    m.def("_last_algo", [](const c10::intrusive_ptr<c10d::Backend>& pg) {
+        auto* p = dynamic_cast<mccl::ProcessGroupMCCL*>(pg.get());
+        return p ? p->lastAlgo() : -1;
+    });
+
+    m.def("_test_progress_order", &progress_order, py::arg("n"), py::arg("throw_mask") = 0,
+          py::arg("use_destructor") = false, py::call_guard<py::gil_scoped_release>());
+    m.def("_test_progress_submit_latency_us", &progress_submit_latency_us,
+          py::call_guard<py::gil_scoped_release>());
+    m.def("_test_work", &work_probe, py::arg("mode"), py::arg("wait_ms") = 1000,
+          py::call_guard<py::gil_scoped_release>());
+    m.def("_test_mesh", &mesh_probe, py::arg("world"), py::arg("rounds") = 3, py::arg("absent") = -1,
+          py::arg("timeout_ms") = 2000, py::arg("leader_throws") = false,
+          py::call_guard<py::gil_scoped_release>());
+}

@@ -443,19 +443,20 @@ int mcclx_allreduce_replay(mcclx_ctx* ctx, const mcclx_replay* r) {
     return replay_fused(ctx, r, L);
 }
 
-int mcclx_reduce_scatter_replay(mcclx_ctx* ctx, int world, void* const* outs,
-                                const void* const* ins, int dtype, uint64_t chunk_numel, int op,
+int mcclx_reduce_scatter_shares(mcclx_ctx* ctx, int world, void* const* outs,
+                                const void* const* shares, int dtype, uint64_t chunk_numel, int op,
                                 int mode, int acc) {
-    if (!ctx || !outs || !ins || world < 1) return bad("reduce_scatter: bad argument");
+    if (!ctx || !outs || !shares || world < 1) return bad("reduce_scatter: bad argument");
+    auto share = [&](int r, int p) { return shares[(size_t)r * (size_t)world + (size_t)p]; };
     const uint64_t cb = chunk_numel * esize(dtype);
-    if (world == 1) return mcclx_copy(ctx, outs[0], ins[0], cb);  // ProcessGroupMCCL.cpp:333-337
+    if (world == 1) return mcclx_copy(ctx, outs[0], share(0, 0), cb);  // ProcessGroupMCCL.cpp:333-337
     bool binary_only = (op != MCCLX_SUM && op != MCCLX_AVG) || dtype == MCCLX_F16;
     bool fused = mode == MCCLX_REPLAY_FUSED && world <= MCCLX_MAX_INPUTS;
     if (!fused) {
         for (int r = 0; r < world; ++r) {  // :357, :378-386
-            TRY(mcclx_copy(ctx, outs[r], at(ins[r], (uint64_t)r * cb), cb));
+            TRY(mcclx_copy(ctx, outs[r], share(r, r), cb));
             for (int p = 0; p < world; ++p)
-                if (p != r) TRY(mcclx_reduce(ctx, outs[r], at(ins[p], (uint64_t)r * cb), dtype, chunk_numel, op));
+                if (p != r) TRY(mcclx_reduce(ctx, outs[r], share(r, p), dtype, chunk_numel, op));
             if (op == MCCLX_AVG)
                 TRY(mcclx_scale(ctx, outs[r], dtype, chunk_numel, 1.0 / (double)world, MCCLX_SCALE_TENSOR));
         }
@@ -468,7 +469,7 @@ int mcclx_reduce_scatter_replay(mcclx_ctx* ctx, int world, void* const* outs,
     p.k = world;
     p.topo = MCCLX_TOPO_FOLD;
     p.op = op;
-    p.acc = acc;
+    p.acc = binary_only ? MCCLX_ACC_STEP : acc;
     p.scale_mode = (op == MCCLX_AVG) ? MCCLX_SCALE_TENSOR : MCCLX_SCALE_NONE;  // metal_scale_inplace
     p.scale = 1.0 / (double)world;
     std::vector<mcclx_seg> segs((size_t)world);
@@ -476,13 +477,23 @@ int mcclx_reduce_scatter_replay(mcclx_ctx* ctx, int world, void* const* outs,
         memset(&segs[r], 0, sizeof(mcclx_seg));
         segs[r].out = outs[r];
         segs[r].count = chunk_numel;
-        segs[r].in[0] = at(ins[r], (uint64_t)r * cb);  // own share first (:357)
+        segs[r].in[0] = share(r, r);  // own share first (:357)
         int j = 1;
         for (int q = 0; q < world; ++q)
-            if (q != r) segs[r].in[j++] = at(ins[q], (uint64_t)r * cb);  // ascending peers (:379-383)
+            if (q != r) segs[r].in[j++] = share(r, q);  // ascending peers (:379-383)
     }
-    if (binary_only) p.acc = MCCLX_ACC_STEP;
     return fold_any(ctx, p, segs);
+}
+
+int mcclx_reduce_scatter_replay(mcclx_ctx* ctx, int world, void* const* outs,
+                                const void* const* ins, int dtype, uint64_t chunk_numel, int op,
+                                int mode, int acc) {
+    if (!ctx || !outs || !ins || world < 1) return bad("reduce_scatter: bad argument");
+    const uint64_t cb = chunk_numel * esize(dtype);
+    std::vector<const void*> shares((size_t)world * (size_t)world);
+    for (int r = 0; r < world; ++r)
+        for (int p = 0; p < world; ++p) shares[(size_t)r * world + p] = at(ins[p], (uint64_t)r * cb);
+    return mcclx_reduce_scatter_shares(ctx, world, outs, shares.data(), dtype, chunk_numel, op, mode, acc);
 }
 
 int mcclx_allgather_replay(mcclx_ctx* ctx, int world, void* const* outs, const void* const* ins,

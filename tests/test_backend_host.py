@@ -1,0 +1,95 @@
+"""Host-side behaviour of the c10d backend pieces, no GPU needed: the FIFO
+engine (the reference's tests/internal/test_progress.cpp cases, and the
+reference's own engine from oracle/_ref run on the same cases), the Work
+object (csrc/backend/WorkMCCL.cpp), the in-process mesh, registration."""
+import ctypes as C
+import datetime
+
+import pytest
+
+from oracle import oracle as orc
+
+
+@pytest.fixture(scope="module")
+def CX():
+    from mccl_amd import _C
+    return _C
+
+
+# ---- Progress: tests/internal/test_progress.cpp:12-63 --------------------
+
+def test_fifo_order_across_many_tasks(CX):
+    assert CX._test_progress_order(100, 0, False) == list(range(100))
+
+
+def test_destructor_drains_the_queue(CX):
+    assert CX._test_progress_order(50, 0, True) == list(range(50))
+
+
+def test_exception_does_not_poison_the_engine(CX):
+    assert CX._test_progress_order(3, 0b001, False) == [1, 2]
+    assert CX._test_progress_order(10, 0b1000010000, False) == [0, 1, 2, 3, 5, 6, 7, 8]
+
+
+def test_submit_does_not_wait_for_a_running_task(CX):
+    assert CX._test_progress_submit_latency_us() < 1000
+
+
+def test_same_observable_order_as_the_reference_engine(CX):
+    R = orc.ref_lib()
+    if R is None:
+        pytest.skip("oracle/_ref not built (reference checkout absent)")
+    for n, mask in ((100, 0), (7, 0b0101010), (64, 0xF0F0F0F0F0F0F0F0)):
+        buf = (C.c_int * n)()
+        k = R.ref_progress_order(n, mask, buf)
+        assert CX._test_progress_order(n, mask, False) == list(buf[:k])
+
+
+# ---- WorkMCCL: csrc/backend/WorkMCCL.cpp:46-104 --------------------------------
+
+def test_work_completion_states(CX):
+    assert CX._test_work("finish", 1000) == (True, True, "")
+    done, ok, msg = CX._test_work("fail", 1000)
+    assert done and not ok and msg == "[MCCL] engine task failed"      # wait() rethrows (:57-59)
+    done, ok, msg = CX._test_work("sync_cb_throws", 1000)
+    assert done and not ok and msg == "[MCCL] drain failed"            # finish() -> sync cb throws (:71-78)
+    assert CX._test_work("late", 2000) == (True, True, "")
+    assert CX._test_work("never", 50) == (False, False, "timeout")     # wait(timeout) returns false (:51-55)
+
+
+# ---- in-process mesh ----------------------------------------------------------
+
+def test_mesh_meets_every_round_with_slots_by_rank(CX):
+    assert CX._test_mesh(4, 5, -1, 5000, False) == ["ok:5"] * 4
+    assert CX._test_mesh(1, 3, -1, 5000, False) == ["ok:3"]
+
+
+def test_mesh_times_out_when_a_rank_is_missing(CX):
+    out = CX._test_mesh(3, 1, 1, 150, False)
+    assert out[1] == "absent"
+    assert all(o.startswith("[MCCL] Timeout: ") for i, o in enumerate(out) if i != 1)
+
+
+def test_mesh_leader_error_reaches_every_rank(CX):
+    assert CX._test_mesh(3, 2, -1, 5000, True) == ["[MCCL] leader failed"] * 3
+
+
+# ---- registration: mccl/_backend.py:30-75, tests/test_smoke.py:12-14 ---------------
+
+def test_backend_is_registered_and_registration_is_idempotent():
+    import torch.distributed as dist
+    import mccl_amd
+    assert mccl_amd.register() is True and mccl_amd.register() is True
+    assert "mccl" in dist.Backend.backend_list
+    assert dist.Backend.backend_capability["mccl"] == ["cuda"]
+
+
+def test_factory_fails_loudly_without_a_gpu(CX):
+    import torch
+    import torch.distributed as dist
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    with pytest.raises(RuntimeError, match=r"\[MCCL\] no usable GPU"):
+        CX._create_process_group_mccl(dist.HashStore(), 0, 1, datetime.timedelta(seconds=5))
+    with pytest.raises(RuntimeError, match="rank/size invalid"):
+        CX._create_process_group_mccl(dist.HashStore(), 3, 2, datetime.timedelta(seconds=5))

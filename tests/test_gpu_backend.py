@@ -1,0 +1,299 @@
+"""The c10d surface on the GPU: world-size-1 semantics (the reference's
+tests/test_smoke.py) and N ranks as N threads of one process sharing the GPU,
+checked bit for bit against the oracle's replay of the reference."""
+import datetime
+import os
+import threading
+
+import numpy as np
+import pytest
+import torch
+import torch.distributed as dist
+
+from oracle import oracle as orc
+from oracle.oracle import F32, F16, BF16, SUM, AVG, MIN, MAX, PRODUCT, RING, TREE, BUTTERFLY
+
+pytestmark = pytest.mark.gpu
+
+TIMEOUT = datetime.timedelta(seconds=20)
+OPS = {SUM: dist.ReduceOp.SUM, AVG: dist.ReduceOp.AVG, MIN: dist.ReduceOp.MIN, MAX: dist.ReduceOp.MAX,
+       PRODUCT: dist.ReduceOp.PRODUCT}
+
+
+@pytest.fixture(scope="module")
+def CX():
+    import mccl_amd
+    from mccl_amd import _C
+    return _C
+
+
+@pytest.fixture(scope="module")
+def U():
+    import gpu_util
+    return gpu_util
+
+
+def run_ranks(CX, world, fn):
+    """Create `world` backends over one HashStore, run fn(rank, pg) on one thread per rank."""
+    store = dist.HashStore()
+    out, errs = [None] * world, [None] * world
+
+    def body(r):
+        try:
+            torch.cuda.set_device(0)
+            pg = CX._create_process_group_mccl(store, r, world, TIMEOUT)
+            out[r] = fn(r, pg)
+        except BaseException as e:  # noqa: BLE001
+            errs[r] = e
+
+    ts = [threading.Thread(target=body, args=(r,)) for r in range(world)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join(60)
+    assert not any(t.is_alive() for t in ts), "a rank thread hung"
+    return out, errs
+
+
+# ---- world size 1: tests/test_smoke.py:29-41 -------------------------------------
+
+def test_world_one_is_a_no_op_with_real_work_objects(CX):
+    pg = CX._create_process_group_mccl(dist.HashStore(), 0, 1, TIMEOUT)
+    assert pg.name() == "mccl" and pg.rank() == 0 and pg.size() == 1
+    t = torch.arange(16, dtype=torch.float32, device="cuda")
+    ref = t.clone()
+    w = pg.allreduce([t])
+    assert w.is_completed() and w.is_success() and w.wait()
+    assert torch.equal(t, ref)
+    assert torch.equal(w.get_future().wait()[0], ref)
+    out = torch.zeros(16, device="cuda")
+    assert pg._allgather_base(out, t).wait() and torch.equal(out, ref)
+    out.zero_()
+    assert pg._reduce_scatter_base(out, t).wait() and torch.equal(out, ref)
+    assert pg.barrier().wait()
+    assert pg.broadcast([t]).wait()
+
+
+def test_init_process_group_world_one(CX):
+    if dist.is_initialized():
+        dist.destroy_process_group()
+    dist.init_process_group(backend="mccl", store=dist.HashStore(), rank=0, world_size=1,
+                            timeout=TIMEOUT)
+    try:
+        assert dist.get_backend() == "mccl"
+        t = torch.full((33,), 3.0, device="cuda")
+        dist.all_reduce(t)
+        assert torch.equal(t, torch.full((33,), 3.0, device="cuda"))
+        o = torch.empty(33, device="cuda")
+        dist.all_gather_into_tensor(o, t)
+        assert torch.equal(o, t)
+    finally:
+        dist.destroy_process_group()
+
+
+# ---- N ranks in one process -----------------------------------------------------------
+
+@pytest.mark.parametrize("world", [2, 3, 4])
+@pytest.mark.parametrize("algo_name,algo", [("ring", RING), ("butterfly", BUTTERFLY), ("tree", TREE), (None, None)])
+@pytest.mark.parametrize("wire", [False, True])
+def test_allreduce_threads_bit_exact(CX, U, monkeypatch, world, algo_name, algo, wire):
+    if algo_name:
+        monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", algo_name)
+    else:
+        monkeypatch.delenv("MCCL_ALLREDUCE_ALGO", raising=False)
+    monkeypatch.delenv("MCCL_TREE_BELOW", raising=False)
+    if wire:
+        monkeypatch.setenv("MCCL_WIRE_DTYPE", "bf16")
+    else:
+        monkeypatch.delenv("MCCL_WIRE_DTYPE", raising=False)
+    rng = np.random.default_rng(world * 10 + (algo or 7))
+    cases = [(F32, SUM, 40009), (F32, AVG, 1237), (BF16, SUM, 70001), (F32, SUM, 100003)]
+    xs = {i: [U.rand_values(rng, n, dt, specials=True) for _ in range(world)] for i, (dt, op, n) in enumerate(cases)}
+
+    def fn(r, pg):
+        res, algos = [], []
+        for i, (dt, op, n) in enumerate(cases):
+            t = U.to_dev(xs[i][r], dt)
+            o = dist.AllreduceOptions()
+            o.reduceOp = OPS[op]
+            w = pg.allreduce([t], o)
+            assert w.is_completed() and w.wait()
+            res.append(t)
+            algos.append(CX._last_algo(pg))
+        return res, algos
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for i, (dt, op, n) in enumerate(cases):
+        want = [x.copy() for x in xs[i]]
+        rc, used = orc.pg_allreduce(want, dt, op, wire_bf16=wire, env_algo=algo_name)
+        assert rc == 0
+        for r in range(world):
+            assert out[r][1][i] == used, "algorithm selection differs from the reference's"
+            U.assert_same_bits(out[r][0][i], want[r], dt, f"case {i} rank {r}")
+
+
+def test_allreduce_min_max_product_fp16_and_tensor_lists(CX, U, monkeypatch):
+    monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "butterfly")
+    monkeypatch.delenv("MCCL_WIRE_DTYPE", raising=False)
+    world = 3
+    rng = np.random.default_rng(5)
+    a = [U.rand_values(rng, 5003, F32) for _ in range(world)]
+    b = [U.rand_values(rng, 777, F16) for _ in range(world)]
+
+    def fn(r, pg):
+        res = {}
+        for op in (MIN, MAX, PRODUCT):
+            t1, t2 = U.to_dev(a[r], F32), U.to_dev(b[r], F16)
+            o = dist.AllreduceOptions(); o.reduceOp = OPS[op]
+            pg.allreduce([t1, t2], o).wait()          # a list of tensors is handled one after another
+            res[op] = (t1, t2)
+        return res
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for op in (MIN, MAX, PRODUCT):
+        wa = [x.copy() for x in a]; orc.allreduce(BUTTERFLY, wa, F32, op)
+        wb = [x.copy() for x in b]; orc.allreduce(BUTTERFLY, wb, F16, op)
+        for r in range(world):
+            U.assert_same_bits(out[r][op][0], wa[r], F32, f"op {op}")
+            assert np.array_equal(U.bits(out[r][op][1]), wb[r])
+
+
+@pytest.mark.parametrize("world", [2, 3, 8])
+def test_reduce_scatter_allgather_broadcast_barrier_threads(CX, U, world):
+    rng = np.random.default_rng(world)
+    CH = 4099
+    ins = [U.rand_values(rng, CH * world, BF16) for _ in range(world)]
+    f32 = [U.rand_values(rng, CH * world, F32) for _ in range(world)]
+
+    def fn(r, pg):
+        res = {}
+        din = U.to_dev(ins[r], BF16)
+        out = torch.empty(CH, dtype=torch.bfloat16, device="cuda")
+        o = dist.ReduceScatterOptions(); o.reduceOp = dist.ReduceOp.AVG
+        w = pg._reduce_scatter_base(out, din, o)          # asynchronous: a pending Work comes back
+        assert w.wait()
+        res["rs_base"] = out
+        # list form, fp32, in place over the rank's own share
+        full = U.to_dev(f32[r], F32)
+        shares = [full.narrow(0, p * CH, CH) for p in range(world)]
+        o2 = dist.ReduceScatterOptions(); o2.reduceOp = dist.ReduceOp.SUM
+        assert pg.reduce_scatter([shares[r]], [shares], o2).wait()
+        res["rs_list"] = shares[r].clone()
+        # allgather, both forms
+        g = torch.empty(CH * world, dtype=torch.bfloat16, device="cuda")
+        assert pg._allgather_base(g, out).wait()
+        res["ag_base"] = g
+        outs = [torch.empty(CH, dtype=torch.bfloat16, device="cuda") for _ in range(world)]
+        fut = pg.allgather([outs], [out]).get_future()
+        fut.wait()
+        res["ag_list"] = torch.cat(outs)
+        # broadcast from the last rank, then a barrier
+        b = torch.full((1001,), float(r), device="cuda")
+        bo = dist.BroadcastOptions(); bo.rootRank = world - 1
+        assert pg.broadcast([b], bo).wait()
+        res["bcast"] = b
+        assert pg.barrier().wait()
+        return res
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    want = [np.zeros(CH, dtype=np.uint16) for _ in range(world)]
+    orc.reduce_scatter(want, ins, BF16, AVG)
+    want32 = [np.zeros(CH, dtype=np.float32) for _ in range(world)]
+    orc.reduce_scatter(want32, f32, F32, SUM)
+    cat = np.concatenate(want)
+    for r in range(world):
+        U.assert_same_bits(out[r]["rs_base"], want[r], BF16, "reduce_scatter_base AVG")
+        U.assert_same_bits(out[r]["rs_list"], want32[r], F32, "reduce_scatter list SUM")
+        assert np.array_equal(U.bits(out[r]["ag_base"]), cat)
+        assert np.array_equal(U.bits(out[r]["ag_list"]), cat)
+        assert torch.equal(out[r]["bcast"], torch.full((1001,), float(world - 1), device="cuda"))
+
+
+def test_error_paths(CX, U):
+    world = 2
+
+    def fn(r, pg):
+        msgs = {}
+        try:
+            pg.allreduce([torch.ones(8)])                       # CPU tensor (test_mps_native.py:343-356)
+        except RuntimeError as e:
+            msgs["cpu"] = str(e)
+        try:
+            o = dist.AllreduceOptions(); o.reduceOp = dist.ReduceOp.BAND
+            pg.allreduce([torch.ones(8, device="cuda")], o)
+        except RuntimeError as e:
+            msgs["op"] = str(e)
+        try:
+            pg.allreduce([torch.ones(8, device="cuda", dtype=torch.float64)])
+        except RuntimeError as e:
+            msgs["dtype"] = str(e)
+        try:
+            pg.allreduce([torch.ones(4, 4, device="cuda").t()])
+        except RuntimeError as e:
+            msgs["contig"] = str(e)
+        # sizes that differ between ranks: every rank gets the leader's error
+        try:
+            pg.allreduce([torch.ones(8 + r, device="cuda")])
+        except RuntimeError as e:
+            msgs["mismatch"] = str(e)
+        # asynchronous collectives report through the Work (ProcessGroupMCCL.cpp:60-68)
+        w = pg._reduce_scatter_base(torch.ones(3, device="cuda"), torch.ones(8, device="cuda"))
+        try:
+            w.wait()
+        except RuntimeError as e:
+            msgs["rs_size"] = str(e)
+        assert w.is_completed() and not w.is_success()
+        w = pg.send([torch.ones(3, device="cuda")], 1 - r, 0)
+        try:
+            w.wait()
+        except RuntimeError as e:
+            msgs["send"] = str(e)
+        # the group still works afterwards
+        t = torch.full((5,), float(r + 1), device="cuda")
+        pg.allreduce([t]).wait()
+        msgs["after"] = t.cpu().tolist()
+        return msgs
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for m in out:
+        assert "GPU-only; got cpu tensor" in m["cpu"]
+        assert "Unsupported ReduceOp" in m["op"]
+        assert "No HIP kernel for dtype" in m["dtype"]
+        assert "must be contiguous" in m["contig"]
+        assert "different size or dtype" in m["mismatch"]
+        assert "input size != output * world" in m["rs_size"]
+        assert "not implemented" in m["send"]
+        assert all(s.startswith("[MCCL] ") for k, s in m.items() if k != "after")
+        assert m["after"] == [3.0] * 5
+
+
+def test_reference_collective_vectors(CX):
+    """tests/collectives/test_allreduce.py:11-28 (128 x value rank+1, all ops, f32/f16/bf16)
+    and tests/test_process_group_local.py:162-207 (3 ranks: SUM = 6, AVG = 2)."""
+    world = 3
+    os.environ.pop("MCCL_ALLREDUCE_ALGO", None)
+    os.environ.pop("MCCL_WIRE_DTYPE", None)
+
+    def fn(r, pg):
+        res = {}
+        for dt in (torch.float32, torch.float16, torch.bfloat16):
+            for name, op in (("sum", dist.ReduceOp.SUM), ("avg", dist.ReduceOp.AVG), ("min", dist.ReduceOp.MIN),
+                             ("max", dist.ReduceOp.MAX), ("prod", dist.ReduceOp.PRODUCT)):
+                for n in (128, 1, 3, 7, 33, 997):
+                    t = torch.full((n,), float(r + 1), dtype=dt, device="cuda")
+                    o = dist.AllreduceOptions(); o.reduceOp = op
+                    pg.allreduce([t], o).wait()
+                    res[(dt, name, n)] = t.float().cpu()
+        return res
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    exp = {"sum": 6.0, "avg": 2.0, "min": 1.0, "max": 3.0, "prod": 6.0}
+    for m in out:
+        for (dt, name, n), got in m.items():
+            tol = 1e-4 if dt == torch.float32 else 1e-2            # tests/common.py:53-56
+            assert torch.allclose(got, torch.full((n,), exp[name]), rtol=tol, atol=tol), (dt, name, n)
