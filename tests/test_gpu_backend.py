@@ -260,7 +260,7 @@ def test_error_paths(CX, U):
     out, errs = run_ranks(CX, world, fn)
     assert errs == [None] * world, errs
     for m in out:
-        assert "GPU-only; got cpu tensor" in m["cpu"]
+        assert "GPU-only; got CPU tensor" in m["cpu"]
         assert "Unsupported ReduceOp" in m["op"]
         assert "No HIP kernel for dtype" in m["dtype"]
         assert "must be contiguous" in m["contig"]
