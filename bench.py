@@ -228,6 +228,20 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
     sets = len(tensors)
     steps, warm = max(20, args.steps // 4), 5
 
+    # what a plain copy kernel reaches at the same footprint (39.3 MB in, 39.3 MB out per launch,
+    # cold-rotated) and at 1 GiB: the practical ceiling next to the published 8 TB/s
+    half = numel * 6
+    pool = torch.empty(16 * half, dtype=torch.uint8, device="cuda")
+    ms, _ = measure(lambda i: q.copy(pool.data_ptr() + (2 * (i % 8) + 1) * half, pool.data_ptr() + 2 * (i % 8) * half, half),
+                    steps, warm)
+    out["plain_copy_same_footprint_GBps"] = round(gbs(2 * half, ms / steps), 1)
+    del pool
+    big = torch.empty(4 << 30, dtype=torch.uint8, device="cuda")
+    ms, _ = measure(lambda i: q.copy(big.data_ptr() + (2 * (i % 2) + 1) * (1 << 30), big.data_ptr() + 2 * (i % 2) * (1 << 30), 1 << 30),
+                    10, 2)
+    out["plain_copy_1GiB_GBps"] = round(gbs(2 << 30, ms / 10), 1)
+    del big
+
     # C2 with the bf16 wire copy for the allgather leg also written (14 B/elem)
     ms, _ = measure(lambda i: q.fold(plan, step_segs(i % sets, with_wire_out=True)), steps, warm)
     out["c2_fold_with_wire_out_GBps"] = round(gbs(numel * 14, ms / steps), 1)

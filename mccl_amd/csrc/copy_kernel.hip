@@ -7,17 +7,37 @@
 
 #include "fold_launch.h"
 
+#ifndef MCCLX_TUNE_COPY_U
+#define MCCLX_TUNE_COPY_U 1
+#endif
+#ifndef MCCLX_TUNE_COPY_NT
+#define MCCLX_TUNE_COPY_NT 1  // every byte is touched once: non-temporal loads and stores
+#endif
+
 namespace mcclx {
 namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+#define MCCLX_GLOBAL __attribute__((address_space(1)))
+#if MCCLX_TUNE_COPY_NT
+#define COPY_LD(p) __builtin_nontemporal_load(p)
+#define COPY_ST(p, v) __builtin_nontemporal_store((v), (p))
+#else
+#define COPY_LD(p) (*(p))
+#define COPY_ST(p, v) (*(p) = (v))
+#endif
 // the widest alignment both pointers share decides the packet type
-template <int A> struct __attribute__((packed, aligned(A))) Packet { u32x4 q; };
+template <int A> struct Packet;
+template <> struct Packet<4> { typedef u32x4 type __attribute__((aligned(4))); };
+template <> struct Packet<2> { typedef u32x4 type __attribute__((aligned(2))); };
+template <> struct Packet<1> { typedef u32x4 type __attribute__((aligned(1))); };
 constexpr int kBlock = 256;
-constexpr int kU = 4;
+constexpr int kU = MCCLX_TUNE_COPY_U;
 
 template <int A>
 __global__ void __launch_bounds__(kBlock) copy_kernel(uint8_t* dst, const uint8_t* src, uint64_t nbytes) {
-    using Raw16B = Packet<A>;
+    typedef typename Packet<A>::type V;
+    const MCCLX_GLOBAL uint8_t* gs = (const MCCLX_GLOBAL uint8_t*)src;
+    MCCLX_GLOBAL uint8_t* gd = (MCCLX_GLOBAL uint8_t*)dst;
     const uint64_t P = nbytes / 16;
     const uint64_t span = (uint64_t)kU * kBlock;
     for (uint64_t base = (uint64_t)blockIdx.x * span; base < P; base += (uint64_t)gridDim.x * span) {
@@ -25,20 +45,20 @@ __global__ void __launch_bounds__(kBlock) copy_kernel(uint8_t* dst, const uint8_
             u32x4 v[kU];
 #pragma unroll
             for (int u = 0; u < kU; ++u)
-                v[u] = reinterpret_cast<const Raw16B*>(src + (base + (uint64_t)u * kBlock + threadIdx.x) * 16)->q;
+                v[u] = COPY_LD((const MCCLX_GLOBAL V*)(gs + (base + (uint64_t)u * kBlock + threadIdx.x) * 16));
 #pragma unroll
             for (int u = 0; u < kU; ++u)
-                reinterpret_cast<Raw16B*>(dst + (base + (uint64_t)u * kBlock + threadIdx.x) * 16)->q = v[u];
+                COPY_ST((MCCLX_GLOBAL V*)(gd + (base + (uint64_t)u * kBlock + threadIdx.x) * 16), v[u]);
         } else {
             for (uint64_t p = base + threadIdx.x; p < P; p += kBlock) {
-                u32x4 v = reinterpret_cast<const Raw16B*>(src + p * 16)->q;
-                reinterpret_cast<Raw16B*>(dst + p * 16)->q = v;
+                u32x4 v = COPY_LD((const MCCLX_GLOBAL V*)(gs + p * 16));
+                COPY_ST((MCCLX_GLOBAL V*)(gd + p * 16), v);
             }
         }
     }
     if (blockIdx.x == 0) {
         uint64_t i = P * 16 + threadIdx.x;
-        if (i < nbytes) dst[i] = src[i];
+        if (i < nbytes) gd[i] = gs[i];
     }
 }
 }  // namespace

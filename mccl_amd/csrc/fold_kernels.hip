@@ -39,7 +39,7 @@ namespace {
 
 // Build-time tuning knobs (defaults are the measured best on MI355X).
 #ifndef MCCLX_TUNE_BLOCK
-#define MCCLX_TUNE_BLOCK 256
+#define MCCLX_TUNE_BLOCK 512
 #endif
 #ifndef MCCLX_TUNE_U
 #define MCCLX_TUNE_U 0  // 0: derive from the register budget of the plan
@@ -155,10 +155,12 @@ struct Cfg {
         for (int k = 0; k < K; ++k) r += (in_is_f32(k) || E == 8) ? 4 : 2;
         return r;
     }
-    // packets in flight per lane per iteration
+    // Packets per lane per iteration.  Measured on MI355X: one packet per lane
+    // and one block per tile (no grid-stride looping) streams fastest whenever an
+    // fp32 stream is present; all-16-bit plans gain a little from two.
     static constexpr int U = MCCLX_TUNE_U ? MCCLX_TUNE_U
                              : (TOPO == MCCLX_TOPO_BINOMIAL) ? 1
-                             : (32 / regs_per_pack() >= 2 ? 2 : 1);
+                             : (E == 8 ? 2 : 1);
 };
 
 typedef u32x4 RawPack;  // one packet of one operand: 16 B, or 8 B in .xy (16-bit operand, E = 4)
@@ -479,10 +481,6 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
     return hipGetLastError();
 }
 
-static bool key_in_is_f32(const PlanKey& key, int k) {
-    return key.dtype == MCCLX_F32 || (key.io == MCCLX_IO_OWN_FIRST_F32 && k == 0) ||
-           (key.io == MCCLX_IO_OWN_LAST_F32 && k == key.k - 1);
-}
 static int key_pack_elems(const PlanKey& key) {
     return (key.dtype == MCCLX_F32 || key.io != MCCLX_IO_PURE) ? 4 : 8;
 }
@@ -499,9 +497,7 @@ uint32_t items_for(const PlanKey& k, uint64_t count) {
 int plan_unroll(const PlanKey& key) {
     if (MCCLX_TUNE_U) return MCCLX_TUNE_U;
     if (key.topo == MCCLX_TOPO_BINOMIAL) return 1;
-    int regs = 0;
-    for (int k = 0; k < key.k; ++k) regs += (key_in_is_f32(key, k) || key_pack_elems(key) == 8) ? 4 : 2;
-    return 32 / regs >= 2 ? 2 : 1;
+    return key_pack_elems(key) == 8 ? 2 : 1;
 }
 
 #define MCCLX_K_CASES(W, IO, TOPO, OP, ACC)                                             \
