@@ -155,12 +155,13 @@ struct Cfg {
         for (int k = 0; k < K; ++k) r += (in_is_f32(k) || E == 8) ? 4 : 2;
         return r;
     }
-    // Packets per lane per iteration.  Measured on MI355X: one packet per lane
-    // and one block per tile (no grid-stride looping) streams fastest whenever an
-    // fp32 stream is present; all-16-bit plans gain a little from two.
+    // Packets per lane per iteration.  Measured on MI355X (one block per tile,
+    // no grid-stride looping): one packet per lane streams fastest for folds with
+    // an fp32 stream; all-16-bit plans and the one-input codec passes (encode,
+    // decode), whose lanes move few bytes, gain 4-12 % from two.
     static constexpr int U = MCCLX_TUNE_U ? MCCLX_TUNE_U
                              : (TOPO == MCCLX_TOPO_BINOMIAL) ? 1
-                             : (E == 8 ? 2 : 1);
+                             : ((E == 8 || (K == 1 && IO != MCCLX_IO_PURE)) ? 2 : 1);
 };
 
 typedef u32x4 RawPack;  // one packet of one operand: 16 B, or 8 B in .xy (16-bit operand, E = 4)
@@ -497,7 +498,7 @@ uint32_t items_for(const PlanKey& k, uint64_t count) {
 int plan_unroll(const PlanKey& key) {
     if (MCCLX_TUNE_U) return MCCLX_TUNE_U;
     if (key.topo == MCCLX_TOPO_BINOMIAL) return 1;
-    return key_pack_elems(key) == 8 ? 2 : 1;
+    return (key_pack_elems(key) == 8 || (key.k == 1 && key.io != MCCLX_IO_PURE)) ? 2 : 1;
 }
 
 #define MCCLX_K_CASES(W, IO, TOPO, OP, ACC)                                             \
@@ -552,6 +553,14 @@ hipError_t launch_fold(hipStream_t st, const PlanKey& key, const LaunchParams& l
             return launch_cfg<Cfg<MCCLX_F32, MCCLX_IO_PURE, 3, 0, 0, 0>>(st, lp);
         if (key.dtype == MCCLX_F32 && key.k == 2)
             return launch_cfg<Cfg<MCCLX_F32, MCCLX_IO_PURE, 2, 0, 0, 0>>(st, lp);
+        if (key.dtype == MCCLX_F32 && key.k == 1)
+            return launch_cfg<Cfg<MCCLX_F32, MCCLX_IO_PURE, 1, 0, 0, 0>>(st, lp);
+        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_OUT_F32 && key.k == 1)
+            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_OUT_F32, 1, 0, 0, 0>>(st, lp);
+        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_PURE && key.k == 2)
+            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_PURE, 2, 0, 0, 0>>(st, lp);
+        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_PURE && key.k == 1)
+            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_PURE, 1, 0, 0, 0>>(st, lp);
     }
     return hipErrorInvalidValue;
 #else
