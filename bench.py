@@ -12,7 +12,8 @@ from): per bucket element 4 B own fp32 read + 2 x 2 B bf16 peer reads + 4 B fp32
 write = 12 B  ->  78,643,200 B.
 
 The K timed steps are recorded into one HIP graph and replayed with a single
-submission, so the host's launch cost is not part of the measurement; steps
+submission, so the host's launch cost is not part of the measurement (the
+warm-up replays the same graph, i.e. max(W, K) untimed steps); steps
 rotate over several distinct copies of the workload (> 512 MiB in total) so the
 256 MiB Infinity Cache cannot serve the reads ("cold", the headline); the same
 loop over one copy is reported as "warm".
@@ -34,7 +35,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 CAL_BYTES = 64 << 20   # size of the calibration copy
 # HBM bytes one C2 fold launch moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by the
 # calibration copy (profiles/c2_fold_hbm_traffic_pmc.txt): 1.004 x the algorithmic bytes.
-C2_MEASURED_TRAFFIC_BYTES = 78_948_716
+C2_MEASURED_TRAFFIC_BYTES = 78_948_925
 
 
 def parse():
@@ -137,13 +138,17 @@ def main():
         return ms_dev, (time.perf_counter() - t0) * 1e3
 
     def measure(seg_fn, steps, warmup):
+        """Untimed warm-up, then exactly `steps` timed steps.  The warm-up replays the
+        same recorded graph (so at least `warmup` steps, in whole replays): the first
+        replays of a freshly instantiated graph run about 4 % slower per kernel than
+        later ones, which is a property of the launch path, not of the kernel.  The
+        data stays cold either way: every replay walks all rotating copies again."""
         torch.cuda.synchronize()  # inputs made by torch ops are complete before the queue reads them
-        gw = record(max(1, warmup), seg_fn)
         gk = record(steps, seg_fn)
-        q.graph_launch(gw)
+        for _ in range(max(1, -(-warmup // steps)) if warmup > 0 else 0):
+            q.graph_launch(gk)
         q.drain()
         ms_dev, ms_wall = timed(gk)
-        q.graph_destroy(gw)
         q.graph_destroy(gk)
         return ms_dev, ms_wall
 

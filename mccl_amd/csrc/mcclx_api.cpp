@@ -726,6 +726,8 @@ int mcclx_graph_end(mcclx_ctx* ctx, mcclx_graph** out) {
     g->tables.swap(ctx->capture_tables);
     hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
     if (e == hipSuccess) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+    // stage the launch's kernel arguments on the device now rather than during the first replay
+    if (e == hipSuccess) e = hipGraphUpload(g->exec, ctx->stream);
     if (e != hipSuccess) {
         if (g->graph) (void)hipGraphDestroy(g->graph);
         for (void* t : g->tables) (void)hipFree(t);

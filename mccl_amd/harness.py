@@ -97,12 +97,13 @@ def allreduce_replay(tensors: List[torch.Tensor], op, algo: int, wire_bf16: bool
     r.numel = tensors[0].numel()
     ptrs = _ptr_array([t.data_ptr() for t in tensors])
     r.tensors = ptrs
+    # the scheduler runs the stepwise schedule itself when a fused request cannot be
+    # folded (binary-only ops, fp16, more than MAX_INPUTS ranks): size for both
     need = L.lib().mcclx_replay_workspace_bytes(C.byref(r))
-    # a FUSED request can fall back to STEPWISE inside the scheduler: size for both
-    r2 = L.Replay.from_buffer_copy(r)
-    r2.mode = L.REPLAY_STEPWISE
-    need = max(need, L.lib().mcclx_replay_workspace_bytes(C.byref(r2))) if mode == L.REPLAY_FUSED and (
-        r.op not in (L.SUM, L.AVG) or r.dtype == L.F16 or r.world > L.MAX_INPUTS) else need
+    if mode == L.REPLAY_FUSED:
+        r.mode = L.REPLAY_STEPWISE
+        need = max(need, L.lib().mcclx_replay_workspace_bytes(C.byref(r)))
+        r.mode = mode
     own_ws = None
     if workspace is None:
         own_ws = workspace = Workspace(q, need)

@@ -123,8 +123,8 @@ int orc_pg_allreduce(int world, void* const* bufs, int dtype, int64_t numel, int
 int orc_reduce_scatter(int world, void* const* outs, const void* const* ins, int dtype,
                        int64_t chunk_numel, int op, int threads);
 
-/* NOT the reference: fp32 accumulation with one final rounding, the variant
- * BASELINE config 5 words as "fp32 accumulation and bf16 output". */
+/* NOT the reference: fp32 accumulation with one final rounding ("fp32
+ * accumulation and bf16 output"), kept as a labelled alternative. */
 int orc_reduce_scatter_f32acc(int world, void* const* outs, const void* const* ins,
                               int64_t chunk_numel, int op, int threads);
 

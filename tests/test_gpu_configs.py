@@ -243,3 +243,29 @@ def test_graph_replays_match_eager(env):
         q.drain()
         assert np.array_equal(U.bits(e), want.view(np.uint32)[:3 * n])
     q.graph_destroy(graph)
+
+
+def test_counts_beyond_32_bits(env):
+    """The reference narrows element counts to uint32 (MetalKernels.mm:156-163);
+    here they are 64-bit: one launch over 2^32 + 4099 bf16 elements, checked
+    against the oracle at the start, across the 2^32 boundary and at the ragged end."""
+    K, H, W, L, U = env
+    n = (1 << 32) + 4099
+    g = torch.Generator(device="cuda").manual_seed(9)
+    a = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+    b = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+    step = 1 << 28
+    for lo in range(0, n, step):
+        m = min(step, n - lo)
+        a[lo:lo + m] = torch.randn(m, device="cuda", generator=g).to(torch.bfloat16)
+        b[lo:lo + m] = torch.randn(m, device="cuda", generator=g).to(torch.bfloat16)
+    windows = [(0, 1 << 16), ((1 << 32) - (1 << 15), (1 << 32) + 4099)]
+    keep = [(U.bits(a[lo:hi]).copy(), U.bits(b[lo:hi]).copy()) for lo, hi in windows]
+    K.hip_sync()
+    K.hip_reduce_op_view(a.data_ptr(), b.data_ptr(), L.BF16, n, "sum")
+    for (lo, hi), (wa, wb) in zip(windows, keep):
+        orc.reduce(wa, wb, BF16, SUM, threads=8)
+        assert np.array_equal(U.bits(a[lo:hi]), wa), (lo, hi)
+    # a chunk boundary beyond 2^32 bytes: chunkize offsets are 64-bit too
+    ch = H.chunkize(n, 2, 3)
+    assert ch[2][2] == 2 * ch[2][0] > (1 << 32) and sum(c[1] for c in ch) == n
