@@ -20,6 +20,7 @@ OBJ_DIR = os.path.join(ROOT, "build", "mcclx")
 LIB_PATH = os.path.join(HERE, "libmcclx.so")
 
 SOURCES = ["fold_kernels.hip", "copy_kernel.hip", "mcclx_api.cpp", "mcclx_sched.cpp"]
+FOLD_PARTS = 6  # fold_kernels.hip is compiled once per part (-DMCCLX_PART=n), in parallel
 HEADERS = ["fold_launch.h", "mcclx_internal.h", os.path.join(ROOT, "include", "mcclx.h")]
 
 # -ffp-contract=off / -fno-fast-math: IEEE fp32 add and mul, no FMA fusion, so
@@ -59,14 +60,20 @@ def build(force: bool = True, verbose: bool = False) -> str:
     cc = hipcc()
     procs = []
     objs = []
+    units = []
     for src in SOURCES:
-        obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+        if src == "fold_kernels.hip":
+            units += [(src, f"fold_kernels_part{n}.o", [f"-DMCCLX_PART={n}"]) for n in range(FOLD_PARTS)]
+        else:
+            units.append((src, os.path.splitext(src)[0] + ".o", []))
+    for src, objname, extra in units:
+        obj = os.path.join(OBJ_DIR, objname)
         objs.append(obj)
-        cmd = [cc] + HIPCC_FLAGS + (["-x", "hip"] if src.endswith(".cpp") else []) + \
+        cmd = [cc] + HIPCC_FLAGS + extra + (["-x", "hip"] if src.endswith(".cpp") else []) + \
               ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
-        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        procs.append((objname, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
     for src, p in procs:
         out, _ = p.communicate()
         out = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l)

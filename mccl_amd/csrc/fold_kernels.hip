@@ -482,6 +482,16 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
     return hipGetLastError();
 }
 
+// The kernel template is instantiated for every supported plan.  To keep build
+// times short the instantiations are spread over several translation units:
+// this file is compiled once per part with -DMCCLX_PART=n (or once, with every
+// part, when MCCLX_PART is not given).
+#ifndef MCCLX_PART
+#define MCCLX_PART -1
+#endif
+#define MCCLX_HAS_PART(n) (MCCLX_PART == -1 || MCCLX_PART == (n))
+
+#if MCCLX_HAS_PART(0)
 static int key_pack_elems(const PlanKey& key) {
     return (key.dtype == MCCLX_F32 || key.io != MCCLX_IO_PURE) ? 4 : 8;
 }
@@ -500,6 +510,7 @@ int plan_unroll(const PlanKey& key) {
     if (key.topo == MCCLX_TOPO_BINOMIAL) return 1;
     return (key_pack_elems(key) == 8 || (key.k == 1 && key.io != MCCLX_IO_PURE)) ? 2 : 1;
 }
+#endif  // part 0: host-side mirrors of the kernel configuration
 
 #define MCCLX_K_CASES(W, IO, TOPO, OP, ACC)                                             \
     switch (key.k) {                                                                    \
@@ -514,6 +525,7 @@ int plan_unroll(const PlanKey& key) {
         default: return hipErrorInvalidValue;                                           \
     }
 
+// k < 4 has one shape only (the binomial tree of 2 or 3 ranks is the left fold)
 #define MCCLX_TOPO_CASES(W, IO, OP, ACC)                                                \
     if (key.topo == MCCLX_TOPO_BINOMIAL && key.k >= 4) {                                \
         MCCLX_K_CASES(W, IO, MCCLX_TOPO_BINOMIAL, OP, ACC)                              \
@@ -521,25 +533,36 @@ int plan_unroll(const PlanKey& key) {
         MCCLX_K_CASES(W, IO, MCCLX_TOPO_FOLD, OP, ACC)                                  \
     }
 
-// k <= 2 only (the reference's binary kernels): MIN / MAX / PRODUCT and fp16.
-#define MCCLX_BINARY_CASES(W, OP)                                                                  \
-    switch (key.k) {                                                                               \
-        case 1: return launch_cfg<Cfg<W, MCCLX_IO_PURE, 1, MCCLX_TOPO_FOLD, OP, MCCLX_ACC_STEP>>(st, lp); \
-        case 2: return launch_cfg<Cfg<W, MCCLX_IO_PURE, 2, MCCLX_TOPO_FOLD, OP, MCCLX_ACC_STEP>>(st, lp); \
+// MIN / MAX / PRODUCT: same-dtype operands, rounding after every step
+#define MCCLX_OTHER_OPS(W)                                                              \
+    switch (key.op) {                                                                   \
+        case MCCLX_PRODUCT: MCCLX_TOPO_CASES(W, MCCLX_IO_PURE, MCCLX_PRODUCT, MCCLX_ACC_STEP) \
+        case MCCLX_MIN: MCCLX_TOPO_CASES(W, MCCLX_IO_PURE, MCCLX_MIN, MCCLX_ACC_STEP)   \
+        case MCCLX_MAX: MCCLX_TOPO_CASES(W, MCCLX_IO_PURE, MCCLX_MAX, MCCLX_ACC_STEP)   \
+        default: return hipErrorInvalidValue;                                           \
+    }
+
+#define MCCLX_BF16_IO_CASES(ACC)                                                                   \
+    switch (key.io) {                                                                              \
+        case MCCLX_IO_PURE: MCCLX_TOPO_CASES(MCCLX_BF16, MCCLX_IO_PURE, MCCLX_SUM, ACC)            \
+        case MCCLX_IO_OUT_F32: MCCLX_TOPO_CASES(MCCLX_BF16, MCCLX_IO_OUT_F32, MCCLX_SUM, ACC)      \
+        case MCCLX_IO_OWN_FIRST_F32:                                                               \
+            MCCLX_TOPO_CASES(MCCLX_BF16, MCCLX_IO_OWN_FIRST_F32, MCCLX_SUM, ACC)                   \
+        case MCCLX_IO_OWN_LAST_F32:                                                                \
+            MCCLX_K_CASES(MCCLX_BF16, MCCLX_IO_OWN_LAST_F32, MCCLX_TOPO_FOLD, MCCLX_SUM, ACC)      \
         default: return hipErrorInvalidValue;                                                      \
     }
 
-#define MCCLX_OP_BINARY(W)                                              \
-    switch (key.op) {                                                   \
-        case MCCLX_PRODUCT: MCCLX_BINARY_CASES(W, MCCLX_PRODUCT)        \
-        case MCCLX_MIN: MCCLX_BINARY_CASES(W, MCCLX_MIN)                \
-        case MCCLX_MAX: MCCLX_BINARY_CASES(W, MCCLX_MAX)                \
-        default: return hipErrorInvalidValue;                           \
-    }
+hipError_t launch_part_sum_f32_f16(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
+hipError_t launch_part_sum_bf16_step(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
+hipError_t launch_part_sum_bf16_f32acc(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
+hipError_t launch_part_ops_f32(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
+hipError_t launch_part_ops_f16(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
+hipError_t launch_part_ops_bf16(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
 
-hipError_t launch_fold(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
 #ifdef MCCLX_TUNE_MINIMAL
-    // tuning builds: only the measured configurations, to keep compile times short
+// tuning builds: only the measured configurations, to keep compile times short
+hipError_t launch_fold(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
     if (key.op == MCCLX_SUM && key.acc == MCCLX_ACC_STEP && key.topo == MCCLX_TOPO_FOLD) {
         if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_OWN_FIRST_F32 && key.k == 3)
             return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_OWN_FIRST_F32, 3, 0, 0, 0>>(st, lp);
@@ -563,42 +586,67 @@ hipError_t launch_fold(hipStream_t st, const PlanKey& key, const LaunchParams& l
             return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_PURE, 1, 0, 0, 0>>(st, lp);
     }
     return hipErrorInvalidValue;
+}
 #else
+
+#if MCCLX_HAS_PART(0)
+hipError_t launch_fold(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
     if (key.op != MCCLX_SUM) {
         if (key.io != MCCLX_IO_PURE || key.acc != MCCLX_ACC_STEP) return hipErrorInvalidValue;
         switch (key.dtype) {
-            case MCCLX_F32: MCCLX_OP_BINARY(MCCLX_F32)
-            case MCCLX_F16: MCCLX_OP_BINARY(MCCLX_F16)
-            case MCCLX_BF16: MCCLX_OP_BINARY(MCCLX_BF16)
+            case MCCLX_F32: return launch_part_ops_f32(st, key, lp);
+            case MCCLX_F16: return launch_part_ops_f16(st, key, lp);
+            case MCCLX_BF16: return launch_part_ops_bf16(st, key, lp);
             default: return hipErrorInvalidValue;
         }
     }
-    if (key.dtype == MCCLX_F32) {
-        if (key.io != MCCLX_IO_PURE) return hipErrorInvalidValue;
-        MCCLX_TOPO_CASES(MCCLX_F32, MCCLX_IO_PURE, MCCLX_SUM, MCCLX_ACC_STEP)
-    }
-    if (key.dtype == MCCLX_F16) {
+    if (key.dtype == MCCLX_F32 || key.dtype == MCCLX_F16) {
         if (key.io != MCCLX_IO_PURE || key.acc != MCCLX_ACC_STEP) return hipErrorInvalidValue;
-        MCCLX_BINARY_CASES(MCCLX_F16, MCCLX_SUM)
+        return launch_part_sum_f32_f16(st, key, lp);
     }
     if (key.dtype != MCCLX_BF16) return hipErrorInvalidValue;
-#define MCCLX_IO_CASES(ACC)                                                                        \
-    switch (key.io) {                                                                              \
-        case MCCLX_IO_PURE: MCCLX_TOPO_CASES(MCCLX_BF16, MCCLX_IO_PURE, MCCLX_SUM, ACC)            \
-        case MCCLX_IO_OUT_F32: MCCLX_TOPO_CASES(MCCLX_BF16, MCCLX_IO_OUT_F32, MCCLX_SUM, ACC)      \
-        case MCCLX_IO_OWN_FIRST_F32:                                                               \
-            MCCLX_TOPO_CASES(MCCLX_BF16, MCCLX_IO_OWN_FIRST_F32, MCCLX_SUM, ACC)                   \
-        case MCCLX_IO_OWN_LAST_F32:                                                                \
-            MCCLX_K_CASES(MCCLX_BF16, MCCLX_IO_OWN_LAST_F32, MCCLX_TOPO_FOLD, MCCLX_SUM, ACC)      \
-        default: return hipErrorInvalidValue;                                                      \
-    }
-    if (key.acc == MCCLX_ACC_STEP) {
-        MCCLX_IO_CASES(MCCLX_ACC_STEP)
-    } else {
-        MCCLX_IO_CASES(MCCLX_ACC_F32)
-    }
-    return hipErrorInvalidValue;
-#endif
+    return key.acc == MCCLX_ACC_STEP ? launch_part_sum_bf16_step(st, key, lp)
+                                     : launch_part_sum_bf16_f32acc(st, key, lp);
 }
+
+hipError_t launch_part_sum_f32_f16(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
+    if (key.dtype == MCCLX_F32) {
+        MCCLX_TOPO_CASES(MCCLX_F32, MCCLX_IO_PURE, MCCLX_SUM, MCCLX_ACC_STEP)
+    }
+    MCCLX_TOPO_CASES(MCCLX_F16, MCCLX_IO_PURE, MCCLX_SUM, MCCLX_ACC_STEP)
+}
+#endif
+
+#if MCCLX_HAS_PART(1)
+hipError_t launch_part_sum_bf16_step(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
+    MCCLX_BF16_IO_CASES(MCCLX_ACC_STEP)
+}
+#endif
+
+#if MCCLX_HAS_PART(2)
+hipError_t launch_part_sum_bf16_f32acc(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
+    MCCLX_BF16_IO_CASES(MCCLX_ACC_F32)
+}
+#endif
+
+#if MCCLX_HAS_PART(3)
+hipError_t launch_part_ops_f32(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
+    MCCLX_OTHER_OPS(MCCLX_F32)
+}
+#endif
+
+#if MCCLX_HAS_PART(4)
+hipError_t launch_part_ops_f16(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
+    MCCLX_OTHER_OPS(MCCLX_F16)
+}
+#endif
+
+#if MCCLX_HAS_PART(5)
+hipError_t launch_part_ops_bf16(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
+    MCCLX_OTHER_OPS(MCCLX_BF16)
+}
+#endif
+
+#endif  // MCCLX_TUNE_MINIMAL
 
 }  // namespace mcclx

@@ -197,11 +197,11 @@ int check_plan(const mcclx_plan* p, mcclx::PlanKey* key, float* scale_f, int* ha
         return fail(MCCLX_ERR_INVALID, "plan.topo=%d unknown", p->topo);
     if (p->acc != MCCLX_ACC_STEP && p->acc != MCCLX_ACC_F32)
         return fail(MCCLX_ERR_INVALID, "plan.acc=%d unknown", p->acc);
-    if (op != MCCLX_SUM && (p->k > 2 || p->io != MCCLX_IO_PURE || p->acc != MCCLX_ACC_STEP))
+    if (op != MCCLX_SUM && (p->io != MCCLX_IO_PURE || p->acc != MCCLX_ACC_STEP))
         return fail(MCCLX_ERR_UNSUPPORTED,
-                    "MIN/MAX/PRODUCT run as the reference's binary kernels only (k<=2, PURE, STEP)");
-    if (p->dtype == MCCLX_F16 && (p->k > 2 || p->acc != MCCLX_ACC_STEP))
-        return fail(MCCLX_ERR_UNSUPPORTED, "fp16 runs as the reference's binary kernels only (k<=2)");
+                    "MIN/MAX/PRODUCT fold same-dtype operands with per-step rounding only (PURE, STEP)");
+    if (p->dtype == MCCLX_F16 && p->acc != MCCLX_ACC_STEP)
+        return fail(MCCLX_ERR_UNSUPPORTED, "fp16 folds round after every step (STEP) only");
     if (p->io == MCCLX_IO_OWN_LAST_F32 && p->topo == MCCLX_TOPO_BINOMIAL)
         return fail(MCCLX_ERR_UNSUPPORTED, "the tree reduces into rank 0: own operand is first");
     int acc = (p->dtype == MCCLX_F32) ? MCCLX_ACC_STEP : p->acc;  // fp32 has no rounding to skip

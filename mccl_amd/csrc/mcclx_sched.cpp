@@ -197,29 +197,8 @@ mcclx_plan base_plan(const mcclx_replay* r, const Layout& L, int k) {
     return p;
 }
 
-// MIN / MAX / PRODUCT and fp16 only exist as binary kernels; a k-input fold of
-// those is k-1 launches accumulating into the output (same order, same result).
 int fold_any(mcclx_ctx* ctx, mcclx_plan p, std::vector<mcclx_seg>& segs) {
-    bool binary_only = (p.op != MCCLX_SUM && p.op != MCCLX_AVG) || p.dtype == MCCLX_F16;
-    if (!binary_only || p.k <= 2) return mcclx_fold_batched(ctx, &p, segs.data(), (uint32_t)segs.size());
-    if (p.topo == MCCLX_TOPO_BINOMIAL) return MCCLX_ERR_UNSUPPORTED;  // caller uses STEPWISE
-    const int K = p.k;
-    int scale_mode = p.scale_mode;
-    for (int j = 1; j < K; ++j) {
-        mcclx_plan q = p;
-        q.k = 2;
-        q.scale_mode = (j == K - 1) ? scale_mode : MCCLX_SCALE_NONE;
-        std::vector<mcclx_seg> step(segs.size());
-        for (size_t s = 0; s < segs.size(); ++s) {
-            memset(&step[s], 0, sizeof(mcclx_seg));
-            step[s].out = segs[s].out;
-            step[s].in[0] = (j == 1) ? segs[s].in[0] : segs[s].out;
-            step[s].in[1] = segs[s].in[j];
-            step[s].count = segs[s].count;
-        }
-        TRY(mcclx_fold_batched(ctx, &q, step.data(), (uint32_t)step.size()));
-    }
-    return MCCLX_OK;
+    return mcclx_fold_batched(ctx, &p, segs.data(), (uint32_t)segs.size());
 }
 
 int replay_fused(mcclx_ctx* ctx, const mcclx_replay* r, const Layout& L) {
@@ -423,16 +402,9 @@ int mcclx_allreduce_replay(mcclx_ctx* ctx, const mcclx_replay* r) {
     if (L.total > 0 && (!r->workspace || r->workspace_bytes < L.total)) return bad("workspace too small");
 
     bool fused = r->mode == MCCLX_REPLAY_FUSED && r->world <= MCCLX_MAX_INPUTS;
-    // the binomial tree of the binary-only kernels (MIN/MAX/PRODUCT, fp16) has
-    // no fused form
-    // Also, a chain of binary launches into `out` needs out to be operand 0
-    // (butterfly); the ring's owner is the LAST operand, and the wire codec
-    // mixes fp32 and bf16 operands, which only the SUM fold handles.
-    bool binary_only = (r->op != MCCLX_SUM && r->op != MCCLX_AVG) || L.wdtype == MCCLX_F16;
-    if (fused && binary_only && r->world > 2 &&
-        (r->algo != MCCLX_ALGO_BUTTERFLY || L.wire))
-        fused = false;
-    if (fused && binary_only && L.wire) fused = false;
+    // The wire codec mixes fp32 and bf16 operands, which only the SUM fold
+    // handles; MIN / MAX / PRODUCT over the wire run the stepwise schedule.
+    if (fused && L.wire && r->op != MCCLX_SUM && r->op != MCCLX_AVG) fused = false;
     if (!fused) {
         mcclx_replay s = *r;
         s.mode = MCCLX_REPLAY_STEPWISE;
@@ -450,7 +422,8 @@ int mcclx_reduce_scatter_shares(mcclx_ctx* ctx, int world, void* const* outs,
     auto share = [&](int r, int p) { return shares[(size_t)r * (size_t)world + (size_t)p]; };
     const uint64_t cb = chunk_numel * esize(dtype);
     if (world == 1) return mcclx_copy(ctx, outs[0], share(0, 0), cb);  // ProcessGroupMCCL.cpp:333-337
-    bool binary_only = (op != MCCLX_SUM && op != MCCLX_AVG) || dtype == MCCLX_F16;
+    // MIN / MAX / PRODUCT and fp16 round after every step by definition
+    bool step_only = (op != MCCLX_SUM && op != MCCLX_AVG) || dtype == MCCLX_F16;
     bool fused = mode == MCCLX_REPLAY_FUSED && world <= MCCLX_MAX_INPUTS;
     if (!fused) {
         for (int r = 0; r < world; ++r) {  // :357, :378-386
@@ -469,7 +442,7 @@ int mcclx_reduce_scatter_shares(mcclx_ctx* ctx, int world, void* const* outs,
     p.k = world;
     p.topo = MCCLX_TOPO_FOLD;
     p.op = op;
-    p.acc = binary_only ? MCCLX_ACC_STEP : acc;
+    p.acc = step_only ? MCCLX_ACC_STEP : acc;
     p.scale_mode = (op == MCCLX_AVG) ? MCCLX_SCALE_TENSOR : MCCLX_SCALE_NONE;  // metal_scale_inplace
     p.scale = 1.0 / (double)world;
     std::vector<mcclx_seg> segs((size_t)world);

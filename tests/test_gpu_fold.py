@@ -66,6 +66,37 @@ def test_fold_pure(K, U, k, dtype, binomial):
         U.assert_same_bits(out, want, dtype, f"k={k} dtype={dtype} binomial={binomial} scale={scale}")
 
 
+@pytest.mark.parametrize("k", [2, 3, 5, 8])
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
+@pytest.mark.parametrize("binomial", [False, True])
+def test_fold_other_ops_and_fp16(K, U, k, dtype, binomial):
+    """MIN / MAX / PRODUCT (and fp16 SUM) as one k-input pass == k-1 binary kernels."""
+    rng = np.random.default_rng(1000 + 10 * k + dtype)
+    n = 30011
+    ops = [orc.MIN, orc.MAX, orc.PRODUCT] + ([SUM] if dtype == F16 else [])
+    for op in ops:
+        ins = [U.rand_values(rng, n, dtype, scale=1.0) for _ in range(k)]
+        v = [x.copy() for x in ins]
+        if not binomial:
+            for j in range(1, k):
+                orc.reduce(v[0], v[j], dtype, op)
+        else:
+            mask = 1
+            while mask < k:
+                for r in range(0, k - mask, 2 * mask):
+                    orc.reduce(v[r], v[r + mask], dtype, op)
+                mask <<= 1
+        d = [U.to_dev(x, dtype) for x in ins]
+        out = torch.empty_like(d[0])
+        plan = K.make_plan(dtype, k, op=op, topo=L().TOPO_BINOMIAL if binomial else L().TOPO_FOLD)
+        K._q(None).fold(plan, [K.make_seg(out.data_ptr(), 0, [t.data_ptr() for t in d], n)])
+        K.hip_sync()
+        if dtype == F16:
+            assert np.array_equal(U.bits(out), v[0]), (op, k)
+        else:
+            U.assert_same_bits(out, v[0], dtype, f"op={op} k={k} dtype={dtype} binomial={binomial}")
+
+
 @pytest.mark.parametrize("k", range(1, 9))
 @pytest.mark.parametrize("io", ["out_f32", "own_first", "own_last"])
 @pytest.mark.parametrize("binomial", [False, True])
@@ -181,8 +212,9 @@ def test_plan_validation(K):
     seg = K.make_seg(a.data_ptr(), 0, [a.data_ptr()] * 8, 64)
     for plan, msg in ((K.make_plan(F32, 0), "plan.k=0"), (K.make_plan(F32, 9), "plan.k=9"),
                       (K.make_plan(F32, 2, io=L().IO_OUT_F32), "bf16 wire dtype"),
-                      (K.make_plan(F32, 3, op=orc.MIN), "binary kernels only"),
-                      (K.make_plan(F16, 3), "fp16 runs as"),
+                      (K.make_plan(BF16, 3, op=orc.MIN, io=L().IO_OUT_F32), "PURE, STEP"),
+                      (K.make_plan(BF16, 3, op=orc.MAX, acc=L().ACC_F32), "PURE, STEP"),
+                      (K.make_plan(F16, 3, acc=L().ACC_F32), "fp16 folds round after every step"),
                       (K.make_plan(F32, 2, op=6), "Unsupported ReduceOp: 6"),
                       (K.make_plan(7, 2), "No kernel for dtype")):
         with pytest.raises(MCCLError, match=msg):
