@@ -59,6 +59,8 @@ def main():
 
     import numpy as np
     import torch
+    from mccl_amd.build import ensure_built
+    ensure_built()
     from mccl_amd import _lib as L
     from mccl_amd import kernels as K
     from mccl_amd import harness as H

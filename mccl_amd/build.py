@@ -144,6 +144,12 @@ def build_backend(verbose: bool = False) -> str:
     return out_path
 
 
+def ensure_built() -> None:
+    """Load what is built; build only if nothing is (used by bench.py and the smoke check)."""
+    if not os.path.exists(LIB_PATH):
+        build(force=True)
+
+
 if __name__ == "__main__":
     print(build(force="--force" in sys.argv or needs_build(), verbose=True))
     if "--backend" in sys.argv:

@@ -27,8 +27,10 @@
  *   orc_allreduce_*       hand-derived fold orders per algorithm, all ranks
  *                         bit-identical, exact integer sums, the reference
  *                         tests' rank+1 vectors.
- *   MIN/MAX on NaN, f16 NaN payloads: parity unpinned (Apple GPU behaviour
- *                         under Metal fast-math is not specified).
+ * Parity unpinned: MIN/MAX with a NaN operand or a +0/-0 tie, and fp16 NaN
+ * payloads (Apple GPU behaviour under Metal fast-math is not specified); the
+ * bit pattern of an encoded NaN (0x7FC0 here, as torch's scalar conversion;
+ * torch's AVX path gives 0xFFFF, Metal's cast is unknown).
  */
 #ifndef MCCL_ORACLE_H
 #define MCCL_ORACLE_H

@@ -12,6 +12,22 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
         sys.path.insert(0, p)
 
 
+def _build_if_nothing_is_built():
+    """Tests load what is built; only when the native libraries are absent do they build them."""
+    from mccl_amd import build as b
+    if not os.path.exists(b.LIB_PATH):
+        b.build(force=True)
+    if not os.path.exists(b.backend_path()):
+        b.build_backend()
+    from oracle import oracle as orc
+    if not os.path.exists(orc.LIB_PATH):
+        orc.build()
+
+
+def pytest_sessionstart(session):
+    _build_if_nothing_is_built()
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
