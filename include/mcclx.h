@@ -216,6 +216,20 @@ MCCLX_API int mcclx_graph_destroy(mcclx_ctx* ctx, mcclx_graph* graph);
 MCCLX_API int mcclx_host_alloc(mcclx_ctx* ctx, uint64_t nbytes, void** host_ptr, void** device_ptr);
 MCCLX_API int mcclx_host_free(mcclx_ctx* ctx, void* host_ptr);
 
+/* Staging for memory the host cannot address (HBM), the other way the
+ * reference moves tensors to and from the wire (MPSInterop.mm:365-435):
+ *   stage_for_send   device -> a pinned staging buffer owned by the context;
+ *                    blocks until the bytes are there; *host_ptr stays valid
+ *                    until the next stage_for_send on this context
+ *                    (StagingBuffer, MPSInterop.hpp:45-51).  Source memory that
+ *                    is already host-addressable (mcclx_host_alloc) is returned
+ *                    as is, without a copy ("direct CPU path", :373-376).
+ *   unstage_from_recv host bytes (any host memory) -> device, asynchronously on
+ *                    the reduce queue; pageable sources go through the pinned
+ *                    staging buffer in pipelined chunks (chunked blits, :47-204). */
+MCCLX_API int mcclx_stage_for_send(mcclx_ctx* ctx, const void* device_src, uint64_t nbytes, void** host_ptr);
+MCCLX_API int mcclx_unstage_from_recv(mcclx_ctx* ctx, void* device_dst, const void* host_src, uint64_t nbytes);
+
 /* ---- chunk scheduler -------------------------------------------------------- */
 
 typedef struct {

@@ -16,6 +16,8 @@ back to another implementation.
 """
 import warnings as _warnings
 
+import torch as _torch  # noqa: F401  first: its HIP runtime must be the one libmcclx binds to (see _lib.py)
+
 from ._lib import MCCLError, LIB_PATH  # noqa: F401
 from ._backend import register
 

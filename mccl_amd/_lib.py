@@ -84,6 +84,8 @@ SIGNATURES = {
     "mcclx_graph_destroy": (_i, [_vp, _vp]),
     "mcclx_host_alloc": (_i, [_vp, _u64, _pp, _pp]),
     "mcclx_host_free": (_i, [_vp, _vp]),
+    "mcclx_stage_for_send": (_i, [_vp, _vp, _u64, _pp]),
+    "mcclx_unstage_from_recv": (_i, [_vp, _vp, _vp, _u64]),
     "mcclx_chunkize": (_i, [_i64, _u64, _i, C.POINTER(Chunk)]),
     "mcclx_select_algo": (_i, [C.c_char_p, _i64, _u64, _i64, _i]),
     "mcclx_replay_workspace_bytes": (_u64, [C.POINTER(Replay)]),
@@ -109,6 +111,13 @@ def lib() -> C.CDLL:
     """Load libmcclx.so (once) and type every entry point.  Raises if absent."""
     global _lib
     if _lib is None:
+        # One HIP runtime per process.  PyTorch-ROCm wheels bundle their own
+        # libamdhip64 (file "libamdhip64.so", soname "libamdhip64.so.N") next to the
+        # system's /opt/rocm copy of the same soname.  The dynamic loader reuses an
+        # already loaded library with a matching soname, so torch must be loaded
+        # first: then libmcclx binds to the runtime that owns torch's tensors.  The
+        # other order loads both runtimes and corrupts the heap at exit.
+        import torch  # noqa: F401
         if not os.path.exists(LIB_PATH):
             raise MCCLError(
                 f"[MCCL] native library {LIB_PATH} is missing: build it with "

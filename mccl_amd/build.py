@@ -134,9 +134,12 @@ def build_backend(verbose: bool = False) -> str:
             print(out[-3000:], flush=True)
     out_path = backend_path()
     tmp = out_path + ".tmp"
+    # libmcclx last: its HIP runtime dependency (soname libamdhip64.so.N) must be
+    # resolved after torch's own copy of that library is loaded, so that the
+    # process ends up with ONE runtime (see mccl_amd/_lib.py).
     link = ["g++", "-shared", "-o", tmp] + objs + [
-        "-L" + HERE, "-lmcclx", "-L" + torch_lib, "-ltorch_python", "-ltorch", "-ltorch_cpu", "-ltorch_hip",
-        "-lc10", "-lc10_hip", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib, "-pthread"]
+        "-L" + torch_lib, "-ltorch_python", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip",
+        "-L" + HERE, "-lmcclx", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib, "-pthread"]
     r = subprocess.run(link, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stdout}")

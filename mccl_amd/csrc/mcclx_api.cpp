@@ -87,6 +87,13 @@ struct mcclx_ctx {
     hipEvent_t xev[16] = {};
     int xnext = 0;
     hipStream_t upload_stream = nullptr;  // blocking table uploads while the queue is recording
+    // staging pool (MPSInterop.mm:47-204): one grow-only pinned buffer for sends,
+    // two fixed pinned chunks + events for pipelined receives from pageable memory
+    void* stage_send = nullptr;
+    size_t stage_send_cap = 0;
+    void* stage_recv[2] = {nullptr, nullptr};
+    hipEvent_t stage_recv_done[2] = {nullptr, nullptr};
+    bool stage_recv_pending[2] = {false, false};
 };
 
 namespace {
@@ -487,6 +494,11 @@ int mcclx_destroy(mcclx_ctx* ctx) {
         if (sl.done) (void)hipEventDestroy(sl.done);
     }
     for (auto& kv : ctx->host_allocs) (void)hipHostFree(kv.first);
+    if (ctx->stage_send) (void)hipHostFree(ctx->stage_send);
+    for (int i = 0; i < 2; ++i) {
+        if (ctx->stage_recv[i]) (void)hipHostFree(ctx->stage_recv[i]);
+        if (ctx->stage_recv_done[i]) (void)hipEventDestroy(ctx->stage_recv_done[i]);
+    }
     if (ctx->upload_stream) (void)hipStreamDestroy(ctx->upload_stream);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
@@ -779,6 +791,94 @@ int mcclx_host_alloc(mcclx_ctx* ctx, uint64_t nbytes, void** host_ptr, void** de
     ctx->host_allocs[h] = nbytes;
     *host_ptr = h;
     *device_ptr = d;
+    return MCCLX_OK;
+}
+
+namespace {
+constexpr size_t kRecvChunk = 8u << 20;  // pinned chunk of the pipelined receive path
+
+// Host-addressable?  (pinned allocations of this library or of anyone else; on
+// ROCm a pinned allocation has one address for host and device)
+bool host_visible(const void* p, void** host_alias) {
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    if (attr.type != hipMemoryTypeHost) return false;
+    *host_alias = const_cast<void*>(p);
+    return true;
+}
+}  // namespace
+
+int mcclx_stage_for_send(mcclx_ctx* ctx, const void* device_src, uint64_t nbytes, void** host_ptr) {
+    if (!ctx || !host_ptr) return fail(MCCLX_ERR_INVALID, "stage_for_send: null argument");
+    if (!device_src || nbytes == 0) return fail(MCCLX_ERR_INVALID, "stage_for_send: empty source");
+    REFUSE_WHILE_RECORDING(ctx, "stage_for_send");
+    DeviceGuard guard(ctx->device);
+    void* alias = nullptr;
+    if (host_visible(device_src, &alias)) {  // direct path: no copy
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+        *host_ptr = alias;
+        return MCCLX_OK;
+    }
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    if (ctx->stage_send_cap < nbytes) {
+        if (ctx->stage_send) HIP_TRY(hipHostFree(ctx->stage_send));
+        ctx->stage_send = nullptr;
+        ctx->stage_send_cap = 0;
+        size_t cap = 1u << 20;
+        while (cap < nbytes) cap <<= 1;
+        hipError_t e = hipHostMalloc(&ctx->stage_send, cap, hipHostMallocDefault);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(MCCLX_ERR_NOMEM, "staging buffer of %zu bytes: %s", cap, hipGetErrorString(e));
+        }
+        ctx->stage_send_cap = cap;
+    }
+    HIP_TRY(hipMemcpyAsync(ctx->stage_send, device_src, nbytes, hipMemcpyDeviceToHost, ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    *host_ptr = ctx->stage_send;
+    return MCCLX_OK;
+}
+
+int mcclx_unstage_from_recv(mcclx_ctx* ctx, void* device_dst, const void* host_src, uint64_t nbytes) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    if (nbytes == 0) return MCCLX_OK;
+    if (!device_dst || !host_src) return fail(MCCLX_ERR_INVALID, "unstage_from_recv: null pointer");
+    REFUSE_WHILE_RECORDING(ctx, "unstage_from_recv");
+    DeviceGuard guard(ctx->device);
+    void* alias = nullptr;
+    if (host_visible(host_src, &alias)) {  // pinned source: one asynchronous copy
+        HIP_TRY(hipMemcpyAsync(device_dst, alias, nbytes, hipMemcpyHostToDevice, ctx->stream));
+        return MCCLX_OK;
+    }
+    // pageable source: memcpy into one pinned chunk while the other is in flight
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    for (int i = 0; i < 2; ++i) {
+        if (!ctx->stage_recv[i]) {
+            hipError_t e = hipHostMalloc(&ctx->stage_recv[i], kRecvChunk, hipHostMallocDefault);
+            if (e != hipSuccess) {
+                (void)hipGetLastError();
+                return fail(MCCLX_ERR_NOMEM, "staging chunk: %s", hipGetErrorString(e));
+            }
+            HIP_TRY(hipEventCreateWithFlags(&ctx->stage_recv_done[i], hipEventDisableTiming));
+        }
+    }
+    const char* src = static_cast<const char*>(host_src);
+    char* dst = static_cast<char*>(device_dst);
+    int slot = 0;
+    for (uint64_t off = 0; off < nbytes; off += kRecvChunk, slot ^= 1) {
+        size_t n = (size_t)((nbytes - off) < kRecvChunk ? (nbytes - off) : kRecvChunk);
+        if (ctx->stage_recv_pending[slot]) {
+            HIP_TRY(hipEventSynchronize(ctx->stage_recv_done[slot]));
+            ctx->stage_recv_pending[slot] = false;
+        }
+        memcpy(ctx->stage_recv[slot], src + off, n);
+        HIP_TRY(hipMemcpyAsync(dst + off, ctx->stage_recv[slot], n, hipMemcpyHostToDevice, ctx->stream));
+        HIP_TRY(hipEventRecord(ctx->stage_recv_done[slot], ctx->stream));
+        ctx->stage_recv_pending[slot] = true;
+    }
     return MCCLX_OK;
 }
 

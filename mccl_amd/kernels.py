@@ -12,6 +12,7 @@ hand-written HIP kernel inside libmcclx.so.
 from __future__ import annotations
 
 import ctypes as C
+import sys as _sys
 from typing import Optional, Sequence
 
 import torch
@@ -77,6 +78,10 @@ class ReduceQueue:
             self._h = C.c_void_p()
 
     def __del__(self):
+        # At interpreter shutdown the HIP runtime and torch may already be tearing
+        # down; the process is about to release everything anyway.
+        if _sys is None or _sys.is_finalizing():
+            return
         try:
             self.close()
         except Exception:
@@ -155,6 +160,18 @@ class ReduceQueue:
 
     def host_free(self, host_address: int) -> None:
         L.check(L.lib().mcclx_host_free(self.handle, C.c_void_p(host_address)))
+
+    # -- staging for memory the host cannot address -----------------------------
+    def stage_for_send(self, device_ptr: int, nbytes: int) -> int:
+        """Device bytes -> pinned staging; returns the host address (valid until the
+        next call).  stage_for_send, MPSInterop.mm:365-406."""
+        h = C.c_void_p()
+        L.check(L.lib().mcclx_stage_for_send(self.handle, C.c_void_p(device_ptr), nbytes, C.byref(h)))
+        return h.value
+
+    def unstage_from_recv(self, device_ptr: int, host_ptr: int, nbytes: int) -> None:
+        """Host bytes -> device, asynchronously on the queue.  unstage_from_recv, MPSInterop.mm:408-435."""
+        L.check(L.lib().mcclx_unstage_from_recv(self.handle, C.c_void_p(device_ptr), C.c_void_p(host_ptr), nbytes))
 
     # -- raw launches ----------------------------------------------------
     def fold(self, plan: L.Plan, segs: Sequence[L.Seg]) -> None:

@@ -120,3 +120,20 @@ def test_missing_library_is_loud(L, monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libmcclx.so"))
     with pytest.raises(_lib.MCCLError, match="is missing"):
         _lib.lib()
+
+
+def test_only_one_hip_runtime_is_loaded_whatever_the_import_order():
+    """PyTorch-ROCm wheels bundle a libamdhip64 next to the system's; loading
+    libmcclx before torch used to pull in both (heap corruption at exit)."""
+    import subprocess
+    import sys
+    code = ("import sys; sys.path.insert(0, %r)\n"
+            "import mccl_amd\n"
+            "from mccl_amd import _lib; _lib.lib()\n"
+            "import torch\n"
+            "libs = sorted(set(l.split()[-1] for l in open('/proc/self/maps') if 'libamdhip64' in l))\n"
+            "print('\\n'.join(libs))\n") % ROOT
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    libs = [l for l in out.stdout.strip().splitlines() if l]
+    assert len(libs) == 1, libs
