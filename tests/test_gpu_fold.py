@@ -225,3 +225,101 @@ def test_plan_validation(K):
         K._q(None).fold(K.make_plan(F32, 1), [K.make_seg(0, 0, [a.data_ptr()], 64)])
     with pytest.raises(MCCLError, match="not element aligned"):
         K._q(None).fold(K.make_plan(F32, 1), [K.make_seg(a.data_ptr() + 2, 0, [a.data_ptr()], 8)])
+
+
+@pytest.mark.parametrize("io", ["encode", "decode", "own_first", "own_last"])
+def test_wire_modes_at_odd_element_offsets(K, U, io):
+    """Chunk starts are only element aligned (C2's second chunk starts 8 B past a
+    16-byte boundary in fp32 and 12 B in bf16): every stream gets its own skew."""
+    rng = np.random.default_rng(len(io))
+    n = 20011
+    for skew in ((0, 0, 0, 0), (1, 0, 0, 0), (0, 1, 2, 3), (3, 5, 7, 1), (2, 2, 2, 2), (31, 63, 1, 33)):
+        own = U.rand_values(rng, n + 64, F32, scale=1e-2, specials=True)
+        p1 = U.rand_values(rng, n + 64, BF16, scale=1e-2, specials=True)
+        p2 = U.rand_values(rng, n + 64, BF16, scale=1e-2, specials=True)
+        d_own, d1, d2 = U.to_dev(own, F32), U.to_dev(p1, BF16), U.to_dev(p2, BF16)
+        o32 = torch.zeros(n + 64, dtype=torch.float32, device="cuda")
+        o16 = torch.zeros(n + 64, dtype=torch.bfloat16, device="cuda")
+        so, s1, s2, sd = skew
+        a = own[so:so + n]
+        if io == "encode":
+            plan = K.make_plan(BF16, 1, io=L().IO_OWN_FIRST_F32)
+            seg = K.make_seg(0, o16.data_ptr() + 2 * sd, [d_own.data_ptr() + 4 * so], n)
+            want16 = orc.encode_bf16(a); want32 = None
+        elif io == "decode":
+            plan = K.make_plan(BF16, 1, io=L().IO_OUT_F32)
+            seg = K.make_seg(o32.data_ptr() + 4 * sd, 0, [d1.data_ptr() + 2 * s1], n)
+            want32 = orc.decode_bf16(p1[s1:s1 + n]); want16 = None
+        else:
+            first = io == "own_first"
+            plan = K.make_plan(BF16, 3, io=L().IO_OWN_FIRST_F32 if first else L().IO_OWN_LAST_F32,
+                               scale_mode=L().SCALE_VIEW, scale=1 / 3)
+            peers = [d1.data_ptr() + 2 * s1, d2.data_ptr() + 2 * s2]
+            ins = [d_own.data_ptr() + 4 * so] + peers if first else peers + [d_own.data_ptr() + 4 * so]
+            seg = K.make_seg(o32.data_ptr() + 4 * sd, o16.data_ptr() + 2 * sd, ins, n)
+            want32, want16 = orc.wire_fold_chunk(np.ascontiguousarray(a),
+                                                 [np.ascontiguousarray(p1[s1:s1 + n]), np.ascontiguousarray(p2[s2:s2 + n])],
+                                                 own_last=not first, scale_by=1 / 3, want_wire=True)
+        K._q(None).fold(plan, [seg])
+        K.hip_sync()
+        if want32 is not None:
+            full = np.zeros(n + 64, np.float32); full[sd:sd + n] = want32
+            U.assert_same_bits(o32, full, F32, f"{io} skew {skew}")          # nothing outside the range is touched
+        if want16 is not None:
+            full = np.zeros(n + 64, np.uint16); full[sd:sd + n] = want16
+            assert np.array_equal(U.bits(o16), full), (io, skew)
+
+
+def test_many_table_launches_in_flight(K, U):
+    """More descriptor-table launches than staging slots, queued without draining,
+    with tables of growing size: slots are reused only after their launch finished."""
+    rng = np.random.default_rng(99)
+    q = K._q(None)
+    n = 3001
+    nseg_list = [9, 12, 40, 9, 300, 17, 1000, 10, 64, 9, 2000, 33]
+    total = max(nseg_list) * n
+    a = U.rand_values(rng, total, F32); b = U.rand_values(rng, total, F32)
+    da, db = U.to_dev(a, F32), U.to_dev(b, F32)
+    outs, wants = [], []
+    plan = K.make_plan(F32, 2)
+    K.hip_sync()
+    for nseg in nseg_list:
+        o = torch.zeros(total, device="cuda")
+        outs.append(o)
+        torch.cuda.synchronize()
+        segs = [K.make_seg(o.data_ptr() + 4 * n * i, 0, [da.data_ptr() + 4 * n * i, db.data_ptr() + 4 * n * i], n)
+                for i in range(nseg)]
+        q.fold(plan, segs)                       # no drain between launches
+        w = np.zeros(total, np.float32); w[:nseg * n] = (a + b)[:nseg * n]
+        wants.append(w)
+    q.drain()
+    for o, w in zip(outs, wants):
+        U.assert_same_bits(o, w, F32, "table launch")
+
+
+def test_two_queues_from_two_threads(K, U):
+    """Contexts are independent: two reduce queues driven from two host threads."""
+    import threading
+    rng = np.random.default_rng(5)
+    n = 1_000_003
+    data = [(U.rand_values(rng, n, BF16), U.rand_values(rng, n, BF16)) for _ in range(2)]
+    res = [None, None]
+
+    def work(i):
+        q = K.ReduceQueue(0)
+        a, b = U.to_dev(data[i][0], BF16), U.to_dev(data[i][1], BF16)
+        torch.cuda.synchronize()
+        for _ in range(20):
+            K.hip_reduce_op_view(a.data_ptr(), b.data_ptr(), BF16, n, SUM, queue=q, drain=False)
+        q.drain()
+        res[i] = U.bits(a)
+        q.close()
+
+    ts = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    [t.start() for t in ts]
+    [t.join(60) for t in ts]
+    for i in range(2):
+        want = data[i][0].copy()
+        for _ in range(20):
+            orc.reduce(want, data[i][1], BF16, SUM, threads=4)
+        assert np.array_equal(res[i], want)
