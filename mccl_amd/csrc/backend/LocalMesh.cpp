@@ -53,6 +53,10 @@ void LocalMesh::rendezvous(int rank, Contribution c, std::chrono::milliseconds t
                            "ranks issued different collectives (rank 0 kind " +
                                std::to_string(slots_[0].kind) + ", rank " + std::to_string(r) +
                                " kind " + std::to_string(slots_[static_cast<size_t>(r)].kind) + ")");
+            for (int r = 0; r < world_; ++r)
+                if (!slots_[static_cast<size_t>(r)].error.empty())
+                    throw MCCLError(slots_[static_cast<size_t>(r)].error + " (raised on rank " +
+                                    std::to_string(r) + ")");
             leader(slots_);
         } catch (...) {
             err = std::current_exception();
@@ -79,6 +83,31 @@ void LocalMesh::rendezvous(int rank, Contribution c, std::chrono::milliseconds t
         throw TimeoutError("rank " + std::to_string(rank) + ": a peer timed out in this collective");
     // generation advanced by exactly one: the error (if any) belongs to our collective
     if (last_error_) std::rethrow_exception(last_error_);
+}
+
+void LocalMesh::post(int src, int dst, Parcel p) {
+    MCCL_CHECK(src >= 0 && src < world_ && dst >= 0 && dst < world_, "rank outside the mesh");
+    {
+        std::lock_guard<std::mutex> lk(box_mu_);
+        boxes_[static_cast<size_t>(src) * static_cast<size_t>(world_) + static_cast<size_t>(dst)].push_back(std::move(p));
+    }
+    box_cv_.notify_all();
+}
+
+Parcel LocalMesh::take(int src, int dst, std::chrono::milliseconds timeout) {
+    MCCL_CHECK(src >= 0 && src < world_ && dst >= 0 && dst < world_, "rank outside the mesh");
+    auto& box = boxes_[static_cast<size_t>(src) * static_cast<size_t>(world_) + static_cast<size_t>(dst)];
+    std::unique_lock<std::mutex> lk(box_mu_);
+    auto ready = [&] { return !box.empty(); };
+    if (timeout.count() <= 0) {
+        box_cv_.wait(lk, ready);
+    } else if (!box_cv_.wait_for(lk, timeout, ready)) {
+        throw TimeoutError("rank " + std::to_string(dst) + ": nothing arrived from rank " + std::to_string(src) +
+                           " within " + std::to_string(timeout.count()) + " ms");
+    }
+    Parcel p = std::move(box.front());
+    box.pop_front();
+    return p;
 }
 
 }  // namespace mccl

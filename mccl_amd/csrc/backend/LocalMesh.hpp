@@ -14,6 +14,7 @@
 #include <chrono>
 #include <condition_variable>
 #include <cstdint>
+#include <deque>
 #include <exception>
 #include <functional>
 #include <memory>
@@ -37,13 +38,30 @@ struct Contribution {
     int wire_bf16 = 0;
     int root = 0;
     void* stream = nullptr;        // the rank's producer/consumer HIP stream
+    std::vector<uint64_t> in_off;  // all-to-all: byte offsets (or sizes) of what goes to each peer
+    std::vector<uint64_t> out_off; // all-to-all: byte offsets (or sizes) of what comes from each peer
+    std::string error;             // set when this rank failed its own argument checks: the
+                                   // rank still arrives, and every rank then fails with this
+                                   // message instead of waiting for a peer that never comes
+};
+
+// One point-to-point message (the reference's 8-byte {tag, nbytes} header followed
+// by the payload, ProcessGroupMCCL.cpp:624-628).  `keep` owns the device buffer
+// `data` points into until the receiver has consumed it.
+struct Parcel {
+    int32_t tag = 0;
+    uint64_t nbytes = 0;
+    const void* data = nullptr;
+    std::shared_ptr<void> keep;
 };
 
 class LocalMesh {
 public:
     using Leader = std::function<void(const std::vector<Contribution>&)>;
 
-    explicit LocalMesh(int world) : world_(world), slots_(static_cast<size_t>(world)) {}
+    explicit LocalMesh(int world)
+        : world_(world), slots_(static_cast<size_t>(world)),
+          boxes_(static_cast<size_t>(world) * static_cast<size_t>(world)) {}
 
     // Process-wide registry: ranks of one group find their mesh by the key the
     // group's store hands out.
@@ -61,6 +79,13 @@ public:
     // TimeoutError and poisons the mesh (later calls fail at once).
     void rendezvous(int rank, Contribution c, std::chrono::milliseconds timeout, const Leader& leader);
 
+    // Point-to-point: one FIFO per ordered pair of ranks, as a socket per peer
+    // gives the reference.  post never blocks (the sender has already copied the
+    // payload into a buffer the parcel owns); take blocks until a parcel from
+    // `src` is there or `timeout` passes (TimeoutError; the mesh stays usable).
+    void post(int src, int dst, Parcel p);
+    Parcel take(int src, int dst, std::chrono::milliseconds timeout);
+
 private:
     const int world_;
     std::mutex mu_;
@@ -70,6 +95,10 @@ private:
     uint64_t generation_ = 0;
     std::exception_ptr last_error_;
     bool broken_ = false;
+
+    std::mutex box_mu_;
+    std::condition_variable box_cv_;
+    std::vector<std::deque<Parcel>> boxes_;   // [src * world + dst]
 };
 
 }  // namespace mccl

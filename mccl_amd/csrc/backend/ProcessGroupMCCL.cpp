@@ -20,22 +20,12 @@ namespace mccl {
 namespace {
 
 enum Kind { K_ALLREDUCE = 1, K_BROADCAST, K_ALLGATHER_BASE, K_ALLGATHER, K_REDUCE_SCATTER_BASE,
-            K_REDUCE_SCATTER, K_BARRIER };
+            K_REDUCE_SCATTER, K_BARRIER, K_ALLTOALL_BASE, K_ALLTOALL };
 
 c10::intrusive_ptr<c10d::Work> make_completed(c10d::OpType op, std::vector<at::Tensor> outputs,
                                               const char* title) {
     auto w = c10::make_intrusive<WorkMCCL>(op, std::move(outputs), title);
     w->finish();
-    return w;
-}
-
-c10::intrusive_ptr<c10d::Work> make_unimplemented(c10d::OpType op, std::vector<at::Tensor> outputs,
-                                                  const char* title) {
-    // the reference's make_unimplemented (ProcessGroupMCCL.cpp:38-43)
-    auto w = c10::make_intrusive<WorkMCCL>(op, std::move(outputs), title);
-    w->finishWithException(std::make_exception_ptr(MCCLError(
-        std::string(title) + ": not implemented (byte transport between processes is outside "
-                             "the single-GPU reduce path)")));
     return w;
 }
 
@@ -79,6 +69,17 @@ int reduce_op_code(const c10d::ReduceOp& op) {
 
 }  // namespace
 
+namespace {
+// torch's caching allocator hands out blocks whose earlier users may still be
+// running on the stream the block belongs to (the allocating thread's current
+// stream); the reduce queue is another stream, so it waits for that one before
+// it touches a fresh block.
+void order_after_allocator(mcclx_ctx* ctx, int device) {
+    check_rc(mcclx_queue_wait_stream(
+        ctx, static_cast<void*>(c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(device)).stream())));
+}
+}  // namespace
+
 // One reduce queue and one grow-only scratch buffer per mesh (per group of
 // ranks sharing the GPU).  The scratch replaces the reference's per-call
 // at::empty recv buffers (ProcessGroupMCCL.cpp:152-162).
@@ -96,6 +97,7 @@ struct ProcessGroupMCCL::Shared {
             check_rc(mcclx_queue_drain(ctx));  // nothing may still read the old buffer
             scratch = at::empty({static_cast<int64_t>(nbytes + 256)},
                                 at::TensorOptions().dtype(at::kByte).device(at::kCUDA, device));
+            order_after_allocator(ctx, device);
         }
         auto p = reinterpret_cast<uintptr_t>(scratch.data_ptr());
         return reinterpret_cast<void*>((p + 255) / 256 * 256);
@@ -168,6 +170,24 @@ void* ProcessGroupMCCL::my_stream() const {
 
 void ProcessGroupMCCL::meet(Contribution c, const LocalMesh::Leader& leader) {
     mesh_->rendezvous(getRank(), std::move(c), opts_.timeout, leader);
+}
+
+// Builds this rank's contribution and meets the peers.  A rank whose own
+// argument checks fail still arrives, carrying the message, so that the whole
+// group fails at once (in the reference such a rank simply never sends and its
+// peers block on their sockets).
+void ProcessGroupMCCL::meet_built(int kind, void* stream, const std::function<void(Contribution&)>& build,
+                                  const LocalMesh::Leader& leader) {
+    Contribution c;
+    try {
+        build(c);
+    } catch (const std::exception& e) {
+        c = Contribution{};
+        c.error = e.what();
+    }
+    c.kind = kind;
+    c.stream = stream;
+    meet(std::move(c), leader);
 }
 
 // The allreduce runs on the caller's thread while every other collective runs
@@ -313,16 +333,14 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::broadcast(std::vector<at::Tenso
     void* stream = my_stream();
     return async_submit_(*engine_, ctx_, stream, c10d::OpType::BROADCAST, tensors, "mccl:broadcast",
                          [this, shared, tensors_copy, root, world, stream]() mutable {
-        Contribution c;
-        c.kind = K_BROADCAST;
-        c.root = root;
-        c.stream = stream;
-        for (auto& t : tensors_copy) {
-            check_gpu_(t, "broadcast");
-            c.dst.push_back(t.data_ptr());
-            c.nbytes.push_back(static_cast<uint64_t>(t.nbytes()));
-        }
-        meet(std::move(c), [shared, world](const std::vector<Contribution>& all) {
+        meet_built(K_BROADCAST, stream, [&](Contribution& c) {
+            c.root = root;
+            for (auto& t : tensors_copy) {
+                check_gpu_(t, "broadcast");
+                c.dst.push_back(t.data_ptr());
+                c.nbytes.push_back(static_cast<uint64_t>(t.nbytes()));
+            }
+        }, [shared, world](const std::vector<Contribution>& all) {
             const int root = all[0].root;
             MCCL_CHECK(root >= 0 && root < world, "broadcast: root outside the group");
             for (int r = 0; r < world; ++r) {
@@ -353,18 +371,16 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::_allgather_base(at::Tensor& out
     void* stream = my_stream();
     return async_submit_(*engine_, ctx_, stream, c10d::OpType::_ALLGATHER_BASE, {output_tensor},
                          "mccl:_allgather_base", [this, shared, out, in, world, stream]() mutable {
-        check_gpu_(in, "_allgather_base");
-        check_gpu_(out, "_allgather_base");
-        const uint64_t chunk = static_cast<uint64_t>(in.nbytes());
-        MCCL_CHECK(static_cast<uint64_t>(out.nbytes()) == chunk * static_cast<uint64_t>(world),
-                   "_allgather_base: output size != input * world");
-        Contribution c;
-        c.kind = K_ALLGATHER_BASE;
-        c.stream = stream;
-        c.dst = {out.data_ptr()};
-        c.src = {in.data_ptr()};
-        c.nbytes = {chunk};
-        meet(std::move(c), [shared, world](const std::vector<Contribution>& all) {
+        meet_built(K_ALLGATHER_BASE, stream, [&](Contribution& c) {
+            check_gpu_(in, "_allgather_base");
+            check_gpu_(out, "_allgather_base");
+            const uint64_t chunk = static_cast<uint64_t>(in.nbytes());
+            MCCL_CHECK(static_cast<uint64_t>(out.nbytes()) == chunk * static_cast<uint64_t>(world),
+                       "_allgather_base: output size != input * world");
+            c.dst = {out.data_ptr()};
+            c.src = {in.data_ptr()};
+            c.nbytes = {chunk};
+        }, [shared, world](const std::vector<Contribution>& all) {
             std::vector<void*> outs(static_cast<size_t>(world));
             std::vector<const void*> ins(static_cast<size_t>(world));
             for (int r = 0; r < world; ++r) {
@@ -393,22 +409,20 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allgather(
     void* stream = my_stream();
     return async_submit_(*engine_, ctx_, stream, c10d::OpType::ALLGATHER, input_tensors, "mccl:allgather",
                          [this, shared, outs_copy, ins_copy, world, stream]() mutable {
-        MCCL_CHECK(ins_copy.size() == outs_copy.size(), "allgather: input/output count mismatch");
-        Contribution c;
-        c.kind = K_ALLGATHER;
-        c.stream = stream;
-        for (size_t i = 0; i < ins_copy.size(); ++i) {
-            MCCL_CHECK(static_cast<int>(outs_copy[i].size()) == world, "allgather: output list size != world");
-            check_gpu_(ins_copy[i], "allgather");
-            c.src.push_back(ins_copy[i].data_ptr());
-            c.nbytes.push_back(static_cast<uint64_t>(ins_copy[i].nbytes()));
-            for (auto& o : outs_copy[i]) {
-                check_gpu_(o, "allgather");
-                MCCL_CHECK(o.nbytes() == ins_copy[i].nbytes(), "allgather: output size != input size");
-                c.dst.push_back(o.data_ptr());
+        meet_built(K_ALLGATHER, stream, [&](Contribution& c) {
+            MCCL_CHECK(ins_copy.size() == outs_copy.size(), "allgather: input/output count mismatch");
+            for (size_t i = 0; i < ins_copy.size(); ++i) {
+                MCCL_CHECK(static_cast<int>(outs_copy[i].size()) == world, "allgather: output list size != world");
+                check_gpu_(ins_copy[i], "allgather");
+                c.src.push_back(ins_copy[i].data_ptr());
+                c.nbytes.push_back(static_cast<uint64_t>(ins_copy[i].nbytes()));
+                for (auto& o : outs_copy[i]) {
+                    check_gpu_(o, "allgather");
+                    MCCL_CHECK(o.nbytes() == ins_copy[i].nbytes(), "allgather: output size != input size");
+                    c.dst.push_back(o.data_ptr());
+                }
             }
-        }
-        meet(std::move(c), [shared, world](const std::vector<Contribution>& all) {
+        }, [shared, world](const std::vector<Contribution>& all) {
             for (int r = 0; r < world; ++r) check_rc(mcclx_queue_wait_stream(shared->ctx, all[r].stream));
             const size_t nt = all[0].src.size();
             for (size_t i = 0; i < nt; ++i)
@@ -437,20 +451,18 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::_reduce_scatter_base(at::Tensor
     void* stream = my_stream();
     return async_submit_(*engine_, ctx_, stream, c10d::OpType::_REDUCE_SCATTER_BASE, {output_tensor},
                          "mccl:_reduce_scatter_base", [this, shared, out, in, op, world, stream]() mutable {
-        check_gpu_(in, "_reduce_scatter_base");
-        check_gpu_(out, "_reduce_scatter_base");
-        MCCL_CHECK(static_cast<uint64_t>(in.nbytes()) == static_cast<uint64_t>(out.nbytes()) * world,
-                   "_reduce_scatter_base: input size != output * world");
-        Contribution c;
-        c.kind = K_REDUCE_SCATTER_BASE;
-        c.op = op;
-        c.stream = stream;
-        c.dst = {out.data_ptr()};
-        c.src = {in.data_ptr()};
-        c.numel = {static_cast<uint64_t>(out.numel())};
-        c.dtype = {need_reduce_dtype(out, "_reduce_scatter_base")};
-        MCCL_CHECK(in.scalar_type() == out.scalar_type(), "_reduce_scatter_base: dtype mismatch");
-        meet(std::move(c), [shared, world](const std::vector<Contribution>& all) {
+        meet_built(K_REDUCE_SCATTER_BASE, stream, [&](Contribution& c) {
+            check_gpu_(in, "_reduce_scatter_base");
+            check_gpu_(out, "_reduce_scatter_base");
+            MCCL_CHECK(static_cast<uint64_t>(in.nbytes()) == static_cast<uint64_t>(out.nbytes()) * world,
+                       "_reduce_scatter_base: input size != output * world");
+            c.op = op;
+            c.dst = {out.data_ptr()};
+            c.src = {in.data_ptr()};
+            c.numel = {static_cast<uint64_t>(out.numel())};
+            c.dtype = {need_reduce_dtype(out, "_reduce_scatter_base")};
+            MCCL_CHECK(in.scalar_type() == out.scalar_type(), "_reduce_scatter_base: dtype mismatch");
+        }, [shared, world](const std::vector<Contribution>& all) {
             std::vector<void*> outs(static_cast<size_t>(world));
             std::vector<const void*> ins(static_cast<size_t>(world));
             for (int r = 0; r < world; ++r) {
@@ -488,27 +500,25 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::reduce_scatter(
     void* stream = my_stream();
     return async_submit_(*engine_, ctx_, stream, c10d::OpType::REDUCE_SCATTER, output_tensors,
                          "mccl:reduce_scatter", [this, shared, outs_copy, ins_copy, op, world, stream]() mutable {
-        MCCL_CHECK(outs_copy.size() == ins_copy.size(), "reduce_scatter: count mismatch");
-        Contribution c;
-        c.kind = K_REDUCE_SCATTER;
-        c.op = op;
-        c.stream = stream;
-        for (size_t i = 0; i < outs_copy.size(); ++i) {
-            auto& out = outs_copy[i];
-            auto& ins = ins_copy[i];
-            MCCL_CHECK(static_cast<int>(ins.size()) == world, "reduce_scatter: input list size != world");
-            check_gpu_(out, "reduce_scatter");
-            c.dst.push_back(out.data_ptr());
-            c.numel.push_back(static_cast<uint64_t>(out.numel()));
-            c.dtype.push_back(need_reduce_dtype(out, "reduce_scatter"));
-            for (auto& t : ins) {
-                check_gpu_(t, "reduce_scatter");
-                MCCL_CHECK(t.nbytes() == out.nbytes() && t.scalar_type() == out.scalar_type(),
-                           "reduce_scatter: output size != input chunk size");
-                c.src.push_back(t.data_ptr());
+        meet_built(K_REDUCE_SCATTER, stream, [&](Contribution& c) {
+            MCCL_CHECK(outs_copy.size() == ins_copy.size(), "reduce_scatter: count mismatch");
+            c.op = op;
+            for (size_t i = 0; i < outs_copy.size(); ++i) {
+                auto& out = outs_copy[i];
+                auto& ins = ins_copy[i];
+                MCCL_CHECK(static_cast<int>(ins.size()) == world, "reduce_scatter: input list size != world");
+                check_gpu_(out, "reduce_scatter");
+                c.dst.push_back(out.data_ptr());
+                c.numel.push_back(static_cast<uint64_t>(out.numel()));
+                c.dtype.push_back(need_reduce_dtype(out, "reduce_scatter"));
+                for (auto& t : ins) {
+                    check_gpu_(t, "reduce_scatter");
+                    MCCL_CHECK(t.nbytes() == out.nbytes() && t.scalar_type() == out.scalar_type(),
+                               "reduce_scatter: output size != input chunk size");
+                    c.src.push_back(t.data_ptr());
+                }
             }
-        }
-        meet(std::move(c), [shared, world](const std::vector<Contribution>& all) {
+        }, [shared, world](const std::vector<Contribution>& all) {
             for (int r = 0; r < world; ++r) check_rc(mcclx_queue_wait_stream(shared->ctx, all[r].stream));
             const size_t nt = all[0].dst.size();
             const size_t W = static_cast<size_t>(world);
@@ -537,40 +547,210 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::barrier(const c10d::BarrierOpti
     void* stream = my_stream();
     return async_submit_(*engine_, ctx_, stream, c10d::OpType::BARRIER, {}, "mccl:barrier",
                          [this, stream]() {
-        Contribution c;
-        c.kind = K_BARRIER;
-        c.stream = stream;
-        meet(std::move(c), [](const std::vector<Contribution>&) {});
+        meet_built(K_BARRIER, stream, [](Contribution&) {}, [](const std::vector<Contribution>&) {});
     });
 }
 
 c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::alltoall_base(at::Tensor& output_tensor, at::Tensor& input_tensor,
-                                                               std::vector<int64_t>&, std::vector<int64_t>&,
+                                                               std::vector<int64_t>& output_split_sizes,
+                                                               std::vector<int64_t>& input_split_sizes,
                                                                const c10d::AllToAllOptions&) {
     if (getSize() == 1) {
         output_tensor.copy_(input_tensor);
         return make_completed(c10d::OpType::ALLTOALL_BASE, {output_tensor}, "mccl:alltoall_base");
     }
-    return make_unimplemented(c10d::OpType::ALLTOALL_BASE, {output_tensor}, "mccl:alltoall_base");
+    at::Tensor out = output_tensor, in = input_tensor;
+    auto out_splits = output_split_sizes;
+    auto in_splits = input_split_sizes;
+    const int world = getSize();
+    const int rank = getRank();
+    auto shared = shared_;
+    void* stream = my_stream();
+    return async_submit_(*engine_, ctx_, stream, c10d::OpType::ALLTOALL_BASE, {output_tensor},
+                         "mccl:alltoall_base",
+                         [this, shared, out, in, out_splits, in_splits, world, rank, stream]() mutable {
+        meet_built(K_ALLTOALL_BASE, stream, [&](Contribution& c) {
+            check_gpu_(in, "alltoall_base");
+            check_gpu_(out, "alltoall_base");
+            const uint64_t esize = static_cast<uint64_t>(in.element_size());
+            MCCL_CHECK(esize == static_cast<uint64_t>(out.element_size()), "alltoall_base: dtype mismatch");
+            const size_t W = static_cast<size_t>(world);
+            // byte offsets of the W pieces (ProcessGroupMCCL.cpp:498-521); split sizes
+            // count rows of dim 0, as c10d defines them
+            auto offsets = [&](const at::Tensor& t, const std::vector<int64_t>& splits, const char* what) {
+                std::vector<uint64_t> off(W + 1, 0);
+                if (splits.empty()) {
+                    const uint64_t per = static_cast<uint64_t>(t.numel()) / W * esize;
+                    MCCL_CHECK(per * W == static_cast<uint64_t>(t.nbytes()),
+                               std::string("alltoall_base: ") + what + " not divisible by world");
+                    for (size_t p = 0; p < W; ++p) off[p + 1] = off[p] + per;
+                } else {
+                    MCCL_CHECK(splits.size() == W, std::string("alltoall_base: ") + what + "_split_sizes wrong length");
+                    const uint64_t row = t.dim() > 0 && t.size(0) > 0
+                                             ? static_cast<uint64_t>(t.nbytes()) / static_cast<uint64_t>(t.size(0))
+                                             : esize;
+                    for (size_t p = 0; p < W; ++p) {
+                        MCCL_CHECK(splits[p] >= 0, std::string("alltoall_base: negative ") + what + " split");
+                        off[p + 1] = off[p] + static_cast<uint64_t>(splits[p]) * row;
+                    }
+                    MCCL_CHECK(off[W] == static_cast<uint64_t>(t.nbytes()),
+                               std::string("alltoall_base: ") + what + "_split_sizes do not add up to the tensor");
+                }
+                return off;
+            };
+            c.in_off = offsets(in, in_splits, "input");
+            c.out_off = offsets(out, out_splits, "output");
+            const size_t r = static_cast<size_t>(rank);
+            MCCL_CHECK(c.in_off[r + 1] - c.in_off[r] == c.out_off[r + 1] - c.out_off[r],
+                       "alltoall_base: self chunk size mismatch");
+            c.src = {in.data_ptr()};
+            c.dst = {out.data_ptr()};
+        }, [shared, world](const std::vector<Contribution>& all) {
+            const size_t W = static_cast<size_t>(world);
+            for (size_t r = 0; r < W; ++r) check_rc(mcclx_queue_wait_stream(shared->ctx, all[r].stream));
+            for (size_t r = 0; r < W; ++r)        // sender
+                for (size_t p = 0; p < W; ++p) {  // receiver
+                    const uint64_t slen = all[r].in_off[p + 1] - all[r].in_off[p];
+                    const uint64_t rlen = all[p].out_off[r + 1] - all[p].out_off[r];
+                    MCCL_CHECK(slen == rlen, "alltoall_base: rank " + std::to_string(r) + " sends " +
+                                                 std::to_string(slen) + " bytes to rank " + std::to_string(p) +
+                                                 ", which expects " + std::to_string(rlen));
+                }
+            // A rank may pass the same buffer as input and output (the reference stages
+            // through host memory, so that works there): then the inputs are first
+            // copied aside, since the pieces are moved one after another on the queue.
+            bool aliased = false;
+            uint64_t total_in = 0;
+            std::vector<uint64_t> base(W + 1, 0);
+            for (size_t r = 0; r < W; ++r) {
+                base[r + 1] = base[r] + (all[r].in_off[W] + 255) / 256 * 256;
+                for (size_t q = 0; q < W; ++q) {
+                    auto a = reinterpret_cast<uintptr_t>(all[r].src[0]);
+                    auto b = reinterpret_cast<uintptr_t>(all[q].dst[0]);
+                    if (a < b + all[q].out_off[W] && b < a + all[r].in_off[W]) aliased = true;
+                }
+            }
+            total_in = base[W];
+            char* aside = aliased ? static_cast<char*>(shared->workspace(total_in)) : nullptr;
+            if (aliased)
+                for (size_t r = 0; r < W; ++r)
+                    if (all[r].in_off[W])
+                        check_rc(mcclx_copy(shared->ctx, aside + base[r], all[r].src[0], all[r].in_off[W]));
+            for (size_t r = 0; r < W; ++r)
+                for (size_t p = 0; p < W; ++p) {
+                    const uint64_t len = all[r].in_off[p + 1] - all[r].in_off[p];
+                    if (len == 0) continue;
+                    const char* from = aliased ? aside + base[r] : static_cast<const char*>(all[r].src[0]);
+                    check_rc(mcclx_copy(shared->ctx, static_cast<char*>(all[p].dst[0]) + all[p].out_off[r],
+                                        from + all[r].in_off[p], len));
+                }
+        });
+    });
 }
 
 c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::alltoall(std::vector<at::Tensor>& output_tensors,
                                                           std::vector<at::Tensor>& input_tensors,
                                                           const c10d::AllToAllOptions&) {
+    MCCL_CHECK(static_cast<int>(input_tensors.size()) == getSize() &&
+                   static_cast<int>(output_tensors.size()) == getSize(),
+               "alltoall: list size != world");  // ProcessGroupMCCL.cpp:555-557
     if (getSize() == 1) {
-        MCCL_CHECK(!output_tensors.empty() && !input_tensors.empty(), "alltoall tensors empty");
         output_tensors[0].copy_(input_tensors[0]);
         return make_completed(c10d::OpType::ALLTOALL, output_tensors, "mccl:alltoall");
     }
-    return make_unimplemented(c10d::OpType::ALLTOALL, output_tensors, "mccl:alltoall");
+    auto outs_copy = output_tensors;
+    auto ins_copy = input_tensors;
+    const int world = getSize();
+    auto shared = shared_;
+    void* stream = my_stream();
+    return async_submit_(*engine_, ctx_, stream, c10d::OpType::ALLTOALL, output_tensors, "mccl:alltoall",
+                         [this, shared, outs_copy, ins_copy, world, stream]() mutable {
+        meet_built(K_ALLTOALL, stream, [&](Contribution& c) {
+            for (int p = 0; p < world; ++p) {
+                check_gpu_(ins_copy[static_cast<size_t>(p)], "alltoall");
+                check_gpu_(outs_copy[static_cast<size_t>(p)], "alltoall");
+                c.src.push_back(ins_copy[static_cast<size_t>(p)].data_ptr());
+                c.dst.push_back(outs_copy[static_cast<size_t>(p)].data_ptr());
+                c.in_off.push_back(static_cast<uint64_t>(ins_copy[static_cast<size_t>(p)].nbytes()));    // sizes here
+                c.out_off.push_back(static_cast<uint64_t>(outs_copy[static_cast<size_t>(p)].nbytes()));
+            }
+        }, [shared, world](const std::vector<Contribution>& all) {
+            const size_t W = static_cast<size_t>(world);
+            for (size_t r = 0; r < W; ++r) check_rc(mcclx_queue_wait_stream(shared->ctx, all[r].stream));
+            for (size_t r = 0; r < W; ++r)
+                for (size_t p = 0; p < W; ++p)
+                    MCCL_CHECK(all[r].in_off[p] == all[p].out_off[r],
+                               "alltoall: rank " + std::to_string(r) + " sends " + std::to_string(all[r].in_off[p]) +
+                                   " bytes to rank " + std::to_string(p) + ", which expects " +
+                                   std::to_string(all[p].out_off[r]));
+            for (size_t r = 0; r < W; ++r)
+                for (size_t p = 0; p < W; ++p)
+                    if (all[r].in_off[p])
+                        check_rc(mcclx_copy(shared->ctx, all[p].dst[r], all[r].src[p], all[r].in_off[p]));
+        });
+    });
 }
 
-c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::send(std::vector<at::Tensor>& tensors, int, int) {
-    return make_unimplemented(c10d::OpType::SEND, tensors, "mccl:send");
+// Point-to-point.  The reference writes an 8-byte {tag, nbytes} header and then
+// the payload to the peer's socket (ProcessGroupMCCL.cpp:614-631); the socket
+// buffers what the receiver has not asked for yet.  Here the sender copies the
+// payload into a device buffer owned by the parcel (so the Work completes
+// without waiting for the receiver, and the sender may reuse its tensor), and
+// the receiver copies it out.  All ranks of a mesh share one reduce queue, so
+// the two copies are ordered by the queue itself.
+c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::send(std::vector<at::Tensor>& tensors, int dst_rank, int tag) {
+    MCCL_CHECK(dst_rank >= 0 && dst_rank < getSize() && dst_rank != getRank(), "send: bad dst_rank");
+    auto tensors_copy = tensors;
+    auto shared = shared_;
+    auto mesh = mesh_;
+    const int rank = getRank();
+    return async_submit_(*engine_, ctx_, my_stream(), c10d::OpType::SEND, tensors, "mccl:send",
+                         [shared, mesh, tensors_copy, rank, dst_rank, tag]() mutable {
+        for (auto& t : tensors_copy) {
+            check_gpu_(t, "send");
+            Parcel p;
+            p.tag = static_cast<int32_t>(tag);
+            p.nbytes = static_cast<uint64_t>(t.nbytes());
+            if (p.nbytes) {
+                auto hold = std::make_shared<at::Tensor>(
+                    at::empty({static_cast<int64_t>(p.nbytes)},
+                              at::TensorOptions().dtype(at::kByte).device(at::kCUDA, shared->device)));
+                order_after_allocator(shared->ctx, shared->device);
+                check_rc(mcclx_copy(shared->ctx, hold->data_ptr(), t.data_ptr(), p.nbytes));
+                p.data = hold->data_ptr();
+                p.keep = hold;
+            }
+            mesh->post(rank, dst_rank, std::move(p));
+        }
+    });
 }
 
-c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::recv(std::vector<at::Tensor>& tensors, int, int) {
-    return make_unimplemented(c10d::OpType::RECV, tensors, "mccl:recv");
+c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::recv(std::vector<at::Tensor>& tensors, int src_rank, int tag) {
+    MCCL_CHECK(src_rank >= 0 && src_rank < getSize() && src_rank != getRank(), "recv: bad src_rank");
+    auto tensors_copy = tensors;
+    auto shared = shared_;
+    auto mesh = mesh_;
+    const int rank = getRank();
+    const auto timeout = opts_.timeout;
+    return async_submit_(*engine_, ctx_, my_stream(), c10d::OpType::RECV, tensors, "mccl:recv",
+                         [shared, mesh, tensors_copy, rank, src_rank, tag, timeout]() mutable {
+        for (auto& t : tensors_copy) {
+            check_gpu_(t, "recv");
+            Parcel p = mesh->take(src_rank, rank, timeout);
+            // header checks of the reference (ProcessGroupMCCL.cpp:645-651)
+            MCCL_CHECK(tag < 0 || p.tag == tag, "recv: tag mismatch (expected " + std::to_string(tag) + " got " +
+                                                    std::to_string(p.tag) + ")");
+            MCCL_CHECK(p.nbytes == static_cast<uint64_t>(t.nbytes()),
+                       "recv: size mismatch (expected " + std::to_string(t.nbytes()) + " got " +
+                           std::to_string(p.nbytes) + ")");
+            if (p.nbytes) {
+                check_rc(mcclx_copy(shared->ctx, t.data_ptr(), p.data, p.nbytes));
+                // the parcel's buffer goes back to torch's allocator when `p` dies:
+                // nothing may still be reading it then
+                check_rc(mcclx_queue_drain(shared->ctx));
+            }
+        }
+    });
 }
 
 }  // namespace mccl

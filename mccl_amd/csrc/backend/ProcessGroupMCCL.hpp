@@ -76,6 +76,8 @@ private:
     struct Shared;  // reduce queue + scratch shared by the ranks of one mesh
 
     void meet(Contribution c, const std::function<void(const std::vector<Contribution>&)>& leader);
+    void meet_built(int kind, void* stream, const std::function<void(Contribution&)>& build,
+                    const std::function<void(const std::vector<Contribution>&)>& leader);
     void* my_stream() const;
     void flush_engine_();
 

@@ -246,9 +246,8 @@ def test_error_paths(CX, U):
         except RuntimeError as e:
             msgs["rs_size"] = str(e)
         assert w.is_completed() and not w.is_success()
-        w = pg.send([torch.ones(3, device="cuda")], 1 - r, 0)
         try:
-            w.wait()
+            pg.send([torch.ones(3, device="cuda")], r, 0)          # to itself (ProcessGroupMCCL.cpp:616-617)
         except RuntimeError as e:
             msgs["send"] = str(e)
         # the group still works afterwards
@@ -266,7 +265,7 @@ def test_error_paths(CX, U):
         assert "must be contiguous" in m["contig"]
         assert "different size or dtype" in m["mismatch"]
         assert "input size != output * world" in m["rs_size"]
-        assert "not implemented" in m["send"]
+        assert "send: bad dst_rank" in m["send"]
         assert all(s.startswith("[MCCL] ") for k, s in m.items() if k != "after")
         assert m["after"] == [3.0] * 5
 
@@ -297,3 +296,205 @@ def test_reference_collective_vectors(CX):
         for (dt, name, n), got in m.items():
             tol = 1e-4 if dt == torch.float32 else 1e-2            # tests/common.py:53-56
             assert torch.allclose(got, torch.full((n,), exp[name]), rtol=tol, atol=tol), (dt, name, n)
+
+
+# ---- all-to-all and point-to-point: the reference's tests/collectives/test_alltoall.py
+# ---- and test_p2p.py, with its values ----------------------------------------------
+
+P2P_DTYPES = [torch.float32, torch.float16, torch.bfloat16, torch.int32, torch.int64, torch.uint8]
+
+
+def seed_tensor(rank, n, dtype):
+    """tests/common.py:136-147 of the reference."""
+    if dtype in (torch.int8, torch.uint8):
+        return torch.full((n,), (rank + 1) % 8, dtype=dtype, device="cuda")
+    return torch.full((n,), rank + 1, dtype=dtype, device="cuda")
+
+
+@pytest.mark.parametrize("world", [2, 3, 4])
+def test_alltoall_base_even_uneven_and_in_place(CX, world):
+    CH = 8
+
+    def fn(r, pg):
+        res = {}
+        for dt in P2P_DTYPES:
+            mk = lambda v, n: torch.full((n,), v, dtype=dt, device="cuda")
+            inp = torch.cat([mk((r * 10 + p) % 120, CH) for p in range(world)])
+            out = torch.empty(CH * world, dtype=dt, device="cuda")
+            pg.alltoall_base(out, inp, [], []).wait()
+            res[(dt, "even")] = out.cpu()
+            same = inp.clone()
+            pg.alltoall_base(same, same, [], []).wait()            # test_alltoall.py:19-23
+            res[(dt, "in_place")] = same.cpu()
+            in_sizes = [4 * (r + 1)] * world                        # test_alltoall.py:29-38
+            out_sizes = [4 * (p + 1) for p in range(world)]
+            inp = torch.cat([mk((r * 10 + p) % 120, in_sizes[p]) for p in range(world)])
+            out = torch.empty(sum(out_sizes), dtype=dt, device="cuda")
+            pg.alltoall_base(out, inp, out_sizes, in_sizes).wait()
+            res[(dt, "uneven")] = out.cpu()
+        # rows of a 2-d tensor: split sizes count rows
+        inp = (torch.arange(world * 2 * 5, device="cuda", dtype=torch.float32) + 1000 * r).reshape(world * 2, 5)
+        out = torch.empty_like(inp)
+        pg.alltoall_base(out, inp, [2] * world, [2] * world).wait()
+        res["rows"] = out.cpu()
+        return res
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for r, res in enumerate(out):
+        for dt in P2P_DTYPES:
+            want = torch.cat([torch.full((CH,), (p * 10 + r) % 120, dtype=dt) for p in range(world)])
+            assert torch.equal(res[(dt, "even")], want), (r, dt)
+            assert torch.equal(res[(dt, "in_place")], want), (r, dt)
+            want = torch.cat([torch.full((4 * (p + 1),), (p * 10 + r) % 120, dtype=dt) for p in range(world)])
+            assert torch.equal(res[(dt, "uneven")], want), (r, dt)
+        want = torch.cat([(torch.arange(world * 10, dtype=torch.float32) + 1000 * p).reshape(world * 2, 5)[2 * r:2 * r + 2]
+                          for p in range(world)])
+        assert torch.equal(res["rows"], want)
+
+
+def test_alltoall_list_form_and_size_errors_reach_every_rank(CX):
+    world = 3
+
+    def fn(r, pg):
+        res = {}
+        ins = [torch.full((5 + p,), float(r * 100 + p), device="cuda") for p in range(world)]
+        outs = [torch.empty(5 + r, device="cuda") for p in range(world)]
+        pg.alltoall(outs, ins).wait()
+        res["list"] = [o.cpu() for o in outs]
+        # rank 1 expects more than its peers send: all ranks fail, at once, with one message
+        import time
+        t0 = time.time()
+        out = torch.empty(8 * world + (1 if r == 1 else 0) * world, device="cuda")
+        w = pg.alltoall_base(out, torch.ones(8 * world, device="cuda"), [], [])
+        try:
+            w.wait()
+            res["err"] = None
+        except RuntimeError as e:
+            res["err"] = str(e)
+        # a rank that fails its own argument check does not leave the others waiting
+        w = pg.alltoall_base(torch.empty(9, device="cuda"), torch.ones(9 if r else 10, device="cuda"), [], [])
+        try:
+            w.wait()
+            res["err2"] = None
+        except RuntimeError as e:
+            res["err2"] = str(e)
+        res["secs"] = time.time() - t0
+        t = torch.full((4,), float(r), device="cuda")
+        pg.allreduce([t]).wait()
+        res["after"] = t.cpu().tolist()
+        return res
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for r, res in enumerate(out):
+        for p in range(world):
+            assert torch.equal(res["list"][p], torch.full((5 + r,), float(p * 100 + r)))
+        assert "which expects" in res["err"] or "self chunk size mismatch" in res["err"], res["err"]
+        assert "input not divisible by world" in res["err2"] and "raised on rank 0" in res["err2"], res["err2"]
+        assert res["secs"] < 10                    # far below the group's 20 s timeout
+        assert res["after"] == [3.0] * 4
+
+
+@pytest.mark.parametrize("world", [2, 3, 4])
+def test_send_recv_ring_tags_and_wildcard(CX, world):
+    """test_p2p.py:8-49: even ranks send first, odd ranks receive first."""
+
+    def fn(r, pg):
+        nxt, prv = (r + 1) % world, (r - 1) % world
+        res = {}
+        for dt in P2P_DTYPES:
+            for tag, want_tag in ((0, 0), (7, 7), (12345, 12345), (42, -1)):
+                send_t = seed_tensor(r, 32, dt)
+                recv_t = torch.empty(32, dtype=dt, device="cuda")
+                if r % 2 == 0:
+                    pg.send([send_t], nxt, tag).wait(); pg.recv([recv_t], prv, want_tag).wait()
+                else:
+                    pg.recv([recv_t], prv, want_tag).wait(); pg.send([send_t], nxt, tag).wait()
+                res[(dt, tag)] = recv_t.cpu()
+        return res
+
+    # with an odd ring two neighbouring even ranks both send first; a send completes
+    # without its receiver here, so no order of calls can deadlock
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for r, res in enumerate(out):
+        for (dt, tag), got in res.items():
+            assert torch.equal(got, seed_tensor((r - 1) % world, 32, dt).cpu()), (r, dt, tag)
+
+
+def test_send_recv_order_headers_and_reuse(CX):
+    world = 2
+    n = 1_000_003
+
+    def fn(r, pg):
+        res = {}
+        peer = 1 - r
+        # both ranks send first, several messages, then receive: FIFO per pair
+        msgs = [torch.full((n,), float(10 * r + i), device="cuda") for i in range(3)]
+        works = [pg.send([m], peer, i) for i, m in enumerate(msgs)]
+        [w.wait() for w in works]
+        for m in msgs:
+            m.add_(1000.0)            # a finished send has taken its copy: the tensor is the sender's again
+        got = [torch.empty(n, device="cuda") for _ in range(3)]
+        rw = [pg.recv([g], peer, i) for i, g in enumerate(got)]
+        [w.wait() for w in rw]
+        res["fifo"] = [float(g[0]) for g in got] + [float(g[-1]) for g in got]
+        # header checks (ProcessGroupMCCL.cpp:645-651)
+        pg.send([torch.ones(4, device="cuda")], peer, 5).wait()
+        try:
+            pg.recv([torch.empty(4, device="cuda")], peer, 6).wait()
+        except RuntimeError as e:
+            res["tag"] = str(e)
+        pg.send([torch.ones(4, device="cuda")], peer, 5).wait()
+        try:
+            pg.recv([torch.empty(3, device="cuda")], peer, 5).wait()
+        except RuntimeError as e:
+            res["size"] = str(e)
+        # several tensors in one call
+        a, b = torch.full((7,), 1.0 + r, device="cuda"), torch.full((9,), 5.0 + r, device="cuda", dtype=torch.float16)
+        pg.send([a, b], peer, 1).wait()
+        ra, rb = torch.empty(7, device="cuda"), torch.empty(9, device="cuda", dtype=torch.float16)
+        pg.recv([ra, rb], peer, 1).wait()
+        res["multi"] = (ra.cpu().tolist(), rb.float().cpu().tolist())
+        return res
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for r, res in enumerate(out):
+        p = 1 - r
+        assert res["fifo"] == [10.0 * p + i for i in range(3)] * 2
+        assert "recv: tag mismatch (expected 6 got 5)" in res["tag"]
+        assert "recv: size mismatch (expected 12 got 16)" in res["size"]
+        assert res["multi"] == ([1.0 + p] * 7, [5.0 + p] * 9)
+
+
+def test_recv_times_out_when_nothing_was_sent(CX):
+    store = dist.HashStore()
+    short = datetime.timedelta(seconds=2)
+    msgs = [None, None]
+
+    def body(r):
+        torch.cuda.set_device(0)
+        pg = CX._create_process_group_mccl(store, r, 2, short)
+        if r == 0:
+            try:
+                pg.recv([torch.empty(4, device="cuda")], 1, 0).wait()
+            except RuntimeError as e:
+                msgs[0] = str(e)
+        # the mesh is still usable: a later message arrives
+        if r == 1:
+            import time; time.sleep(3.0)
+            pg.send([torch.full((4,), 9.0, device="cuda")], 0, 3).wait()
+            msgs[1] = "sent"
+        else:
+            t = torch.empty(4, device="cuda")
+            pg.recv([t], 1, 3).wait()
+            msgs.append(t.cpu().tolist())
+
+    ts = [threading.Thread(target=body, args=(r,)) for r in range(2)]
+    [t.start() for t in ts]
+    [t.join(30) for t in ts]
+    assert not any(t.is_alive() for t in ts)
+    assert "Timeout" in msgs[0] and "nothing arrived from rank 1" in msgs[0]
+    assert msgs[2] == [9.0] * 4
