@@ -1,0 +1,166 @@
+"""Long loops over the c10d surface (the reference's tests/test_soak.py:66-188), N ranks as
+N threads on the one GPU.  The reference only checks that nothing hangs or throws; here every
+iteration's result is also checked on the device and the last one bit for bit on the host."""
+import datetime
+import threading
+
+import numpy as np
+import pytest
+import torch
+import torch.distributed as dist
+
+pytestmark = pytest.mark.gpu
+
+TIMEOUT = datetime.timedelta(seconds=30)
+
+
+@pytest.fixture(scope="module")
+def CX():
+    import mccl_amd
+    from mccl_amd import _C
+    return _C
+
+
+def run_ranks(CX, world, fn, join_s=120):
+    store = dist.HashStore()
+    out, errs = [None] * world, [None] * world
+
+    def body(r):
+        try:
+            torch.cuda.set_device(0)
+            pg = CX._create_process_group_mccl(store, r, world, TIMEOUT)
+            out[r] = fn(r, pg)
+        except BaseException as e:  # noqa: BLE001
+            errs[r] = e
+
+    ts = [threading.Thread(target=body, args=(r,)) for r in range(world)]
+    [t.start() for t in ts]
+    [t.join(join_s) for t in ts]
+    assert not any(t.is_alive() for t in ts), "a rank thread hung"
+    assert errs == [None] * world, errs
+    return out
+
+
+def values(seed, rank, n, device="cuda"):
+    """What rank `rank` contributes in iteration `seed`: cheap, deterministic, known to every rank."""
+    g = torch.Generator(device="cpu").manual_seed(seed * 131 + rank)
+    return torch.randn(n, generator=g).to(device)
+
+
+def test_allreduce_loop_two_ranks(CX):
+    """test_soak.py:69-76 (10k x 1024 floats, SUM); 3000 iterations here, each one checked."""
+    def fn(r, pg):
+        bad = torch.zeros((), device="cuda", dtype=torch.int64)
+        base = [values(0, p, 1024) for p in range(2)]
+        for i in range(3000):
+            t = base[r] * float(i + 1)
+            pg.allreduce([t]).wait()
+            want = base[0] * float(i + 1) + base[1] * float(i + 1)      # x0 + x1 in either order
+            bad += (t != want).sum()
+        return int(bad)
+
+    assert run_ranks(CX, 2, fn) == [0, 0]
+
+
+def test_mixed_sizes_and_large_buckets(CX):
+    """test_soak.py:78-98: sizes 64 .. 1 Mi round robin, then 100 MB buckets."""
+    sizes = [64, 1024, 4096, 65536, 262144, 1048576]
+
+    def fn(r, pg):
+        bad = 0
+        for i in range(100):
+            n = sizes[i % len(sizes)]
+            xs = [values(i, p, n) for p in range(2)]
+            t = xs[r].clone()
+            pg.allreduce([t]).wait()
+            bad += int((t != xs[0] + xs[1]).sum())
+        big = [torch.full((25_000_000,), float(p + 1), device="cuda") for p in range(2)]
+        for _ in range(10):
+            t = big[r].clone()
+            pg.allreduce([t]).wait()
+            bad += int((t != 3.0).sum())
+        return bad
+
+    assert run_ranks(CX, 2, fn) == [0, 0]
+
+
+def test_interleaved_collectives(CX):
+    """test_soak.py:100-117: allreduce every iteration, broadcast every 10th, barrier every 50th;
+    the asynchronous ones are waited for late, to let them queue up behind each other."""
+    def fn(r, pg):
+        bad = 0
+        pending = []
+        for i in range(500):
+            xs = [values(i, p, 4096) for p in range(2)]
+            t = xs[r].clone()
+            pg.allreduce([t]).wait()
+            bad += int((t != xs[0] + xs[1]).sum())
+            if i % 10 == 0:
+                b = values(i + 7, 0, 1024) if r == 0 else torch.zeros(1024, device="cuda")
+                pending.append((pg.broadcast([b]), b, values(i + 7, 0, 1024)))
+            if i % 25 == 0:
+                out = torch.empty(2048, device="cuda")
+                pending.append((pg._reduce_scatter_base(out, torch.cat([xs[r], xs[r]])[:4096].contiguous()),
+                                out, (xs[0] + xs[1])[2048 * r:2048 * (r + 1)] if r == 0 else
+                                (xs[0] + xs[1])[2048:4096]))
+            if i % 50 == 0:
+                pending.append((pg.barrier(), None, None))
+            if len(pending) > 8:
+                for w, got, want in pending:
+                    w.wait()
+                    if got is not None:
+                        bad += int((got != want).sum())
+                pending.clear()
+        for w, got, want in pending:
+            w.wait()
+            if got is not None:
+                bad += int((got != want).sum())
+        return bad
+
+    assert run_ranks(CX, 2, fn) == [0, 0]
+
+
+def test_three_ranks_every_op_and_odd_sizes(CX):
+    """test_soak.py:123-188: 3 ranks, SUM loop, the five ops in turn on rank+1, and the
+    sizes that are not multiples of the vector width (fp32 and fp16)."""
+    ops = [dist.ReduceOp.SUM, dist.ReduceOp.MIN, dist.ReduceOp.MAX, dist.ReduceOp.PRODUCT, dist.ReduceOp.AVG]
+    expect = [6.0, 1.0, 3.0, 6.0, 2.0]
+    odd = [1, 3, 5, 7, 9, 11, 13, 15, 17, 31, 33, 63, 65, 127, 129, 255, 257, 511, 513, 1023, 1025]
+
+    def fn(r, pg):
+        bad = 0
+        for i in range(1000):
+            t = torch.full((1024,), float(r + i), device="cuda")
+            pg.allreduce([t]).wait()
+            bad += int((t != float(3 * i + 3)).sum())
+        for i in range(500):
+            o = dist.AllreduceOptions(); o.reduceOp = ops[i % 5]
+            t = torch.ones(256, device="cuda") * (r + 1)
+            pg.allreduce([t], o).wait()
+            bad += int((t != expect[i % 5]).sum())
+        for rep in range(5):
+            for n in odd:
+                for dt in (torch.float32, torch.float16):
+                    t = torch.full((n,), float(r + 1), device="cuda", dtype=dt)
+                    pg.allreduce([t]).wait()
+                    bad += int((t.float() != 6.0).sum())
+        return bad
+
+    assert run_ranks(CX, 3, fn) == [0, 0, 0]
+
+
+def test_groups_come_and_go(CX):
+    """Fifty groups created, used once and dropped: meshes, engines and queues are released."""
+    for i in range(50):
+        world = 2 + i % 3
+
+        def fn(r, pg):
+            t = torch.full((33,), float(r + 1), device="cuda")
+            pg.allreduce([t]).wait()
+            out = torch.empty(33 * world, device="cuda")
+            pg._allgather_base(out, torch.full((33,), float(r), device="cuda")).wait()
+            return float(t[0]), out[::33].cpu().tolist()
+
+        res = run_ranks(CX, world, fn)
+        for r in range(world):
+            assert res[r] == (world * (world + 1) / 2, [float(p) for p in range(world)])
