@@ -253,6 +253,36 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
     ms, _ = measure(lambda i: q.fold(plan, step_segs(i % sets, with_wire_out=True)), steps, warm)
     out["c2_fold_with_wire_out_GBps"] = round(gbs(numel * 14, ms / steps), 1)
 
+    # the same fold with four buckets in ONE launch (the batched entry point): the fixed cost of a
+    # launch (about 2 us of ramp-up and drain) is paid once per 100 MiB instead of once per 25 MiB
+    nb = min(4, sets)
+    ms, _ = measure(lambda i: q.fold(plan, [s for b in range(nb) for s in step_segs((nb * i + b) % sets)]),
+                    max(10, steps // nb), warm)
+    out["c2_fold_4_buckets_per_launch_GBps"] = round(gbs(nb * numel * 12, ms / max(10, steps // nb)), 1)
+
+    # C2 with the peers' bf16 chunks left where a NIC or a host transport puts them: pinned host
+    # memory, read by the kernel through its device alias (4 B/elem cross PCIe, 8 B/elem stay in HBM)
+    pin = []
+    try:
+        alias = []
+        for p in range(world):
+            hptr, dptr = q.host_alloc(numel * 2)
+            pin.append(hptr)
+            alias.append(dptr)
+            q.copy(dptr, wires[0][p].data_ptr(), numel * 2)
+        q.drain()
+        psegs = []
+        for R, (start, cnt, _, _) in enumerate(chunks):
+            own = tensors[0][R].data_ptr() + start * 4
+            psegs.append(K.make_seg(own, 0, [own] + [alias[p] + start * 2 for p in range(world) if p != R], cnt))
+        ms, _ = measure(lambda i: q.fold(plan, psegs), 10, 2)
+        out["c2_fold_peers_in_pinned_host_us"] = round(ms / 10 * 1e3, 1)
+        out["c2_fold_peers_in_pinned_host_PCIe_GBps"] = round(gbs(numel * 4, ms / 10), 1)
+        out["c2_fold_peers_in_pinned_host_GBps"] = round(gbs(numel * 12, ms / 10), 1)
+    finally:
+        for hptr in pin:
+            q.host_free(hptr)
+
     # encode leg: 3 ranks x (4 B read + 2 B write) per element
     def enc(i):
         s = i % sets

@@ -427,34 +427,55 @@ __global__ void __launch_bounds__(kBlock) fold_few_kernel(FewArgs a) {
                     (uint64_t)gridDim.x * span, blockIdx.x == 0);
 }
 
-// Persistent blocks over a descriptor table in device memory: work item w is
-// tile (w - first_item[seg]) of segment seg; a block takes items
-// blockIdx.x, blockIdx.x + gridDim.x, ...  The loop bound is fixed at launch,
-// so every wave exits.
+// A value that is the same in every lane, moved to scalar registers.  The
+// compiler cannot always prove it (a quotient comes out of the vector ALU), and
+// a descriptor kept in vector registers costs the kernel a quarter of its
+// resident blocks.
+__device__ __forceinline__ uint32_t uni32(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ uint64_t uni64(uint64_t v) {
+    return ((uint64_t)uni32((uint32_t)(v >> 32)) << 32) | uni32((uint32_t)v);
+}
+template <class P>
+__device__ __forceinline__ P* uniptr(P* p) {
+    return reinterpret_cast<P*>(uni64(reinterpret_cast<uint64_t>(p)));
+}
+
+// Blocks over a descriptor table in device memory: work item w is tile
+// (w - first_item[seg]) of segment seg; a block takes items blockIdx.x,
+// blockIdx.x + gridDim.x, ...  (one item per block unless the grid is capped).
+// The loop bound is fixed at launch, so every wave exits.  total_items < 2^31
+// (checked by the host).
 template <class C>
 __global__ void __launch_bounds__(kBlock) fold_table_kernel(TableArgs a) {
     const uint64_t span = (uint64_t)C::U * kBlock;
-    for (uint64_t w = blockIdx.x; w < a.total_items; w += gridDim.x) {
-        uint32_t seg;
-        uint64_t tile;
-        if (a.uniform_items) {
-            seg = (uint32_t)(w / a.uniform_items);
-            tile = w - (uint64_t)seg * a.uniform_items;
+    const uint32_t total = (uint32_t)a.total_items;
+    const uint32_t uniform = (uint32_t)a.uniform_items;
+    for (uint32_t w = blockIdx.x; w < total; w += gridDim.x) {
+        uint32_t seg, tile;
+        if (uniform) {
+            seg = w / uniform;
+            tile = w - seg * uniform;
         } else {
             uint32_t lo = 0, hi = a.nseg;  // first_item[lo] <= w < first_item[hi]
             while (hi - lo > 1) {
                 uint32_t mid = (lo + hi) >> 1;
-                if (a.first_item[mid] <= w) lo = mid; else hi = mid;
+                if ((uint32_t)a.first_item[mid] <= w) lo = mid; else hi = mid;
             }
             seg = lo;
-            tile = w - a.first_item[seg];
+            tile = w - (uint32_t)a.first_item[seg];
         }
-        // w depends on blockIdx only, so the segment is the same for every lane:
-        // say so, and its descriptor is fetched with scalar loads
-        seg = __builtin_amdgcn_readfirstlane(seg);
-        SegArgs s = a.segs[seg];
+        // w depends on blockIdx only, so segment and tile are the same for every lane
+        seg = uni32(seg);
+        tile = uni32(tile);
+        const SegArgs* __restrict__ d = a.segs + seg;
+        SegArgs s;
+        s.out = uniptr(d->out);
+        s.wire_out = uniptr(d->wire_out);
+#pragma unroll
+        for (int k = 0; k < MCCLX_MAX_INPUTS; ++k) s.in[k] = (k < C::K) ? uniptr(d->in[k]) : nullptr;
+        s.count = uni64(d->count);
         // one tile: packets [tile*span, tile*span + span); tile 0 also owns the tail
-        fold_segment<C>(s, a.scale, a.has_scale != 0, tile * span, ~0ull >> 1, tile == 0);
+        fold_segment<C>(s, a.scale, a.has_scale != 0, (uint64_t)tile * span, ~0ull >> 1, tile == 0);
     }
 }
 

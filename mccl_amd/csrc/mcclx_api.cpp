@@ -70,6 +70,7 @@ struct mcclx_ctx {
     bool own_stream = false;
     int cus = 0;
     uint32_t max_blocks = 0;
+    uint32_t few_max = mcclx::kFewSegs;  // segments up to which descriptors travel in the kernel arguments
     bool validate = false;
     bool batch_active = false;
     std::string batch_label;
@@ -324,7 +325,7 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
 
     mcclx::LaunchParams lp;
     lp.max_blocks = ctx->max_blocks;
-    if (nseg <= (uint32_t)mcclx::kFewSegs) {
+    if (nseg <= ctx->few_max) {
         mcclx::FewArgs a;
         memset(&a, 0, sizeof a);
         for (uint32_t s = 0; s < nseg; ++s) memcpy(&a.seg[s], &segs[s], sizeof(mcclx_seg));
@@ -357,6 +358,7 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
         }
         pre[nseg] = total;
         if (total == 0) return MCCLX_OK;
+        if (total >> 31) return fail(MCCLX_ERR_INVALID, "fold: more than 2^31 work items in one launch");
         void* dev = nullptr;
         HIP_TRY(hipMalloc(&dev, host.size()));
         // not the legacy stream: that one may not be touched while another stream records
@@ -397,6 +399,7 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
     }
     pre[nseg] = total;
     if (total == 0) return MCCLX_OK;
+    if (total >> 31) return fail(MCCLX_ERR_INVALID, "fold: more than 2^31 work items in one launch");
     HIP_TRY(hipMemcpyAsync(sl.dev, sl.host, seg_bytes + pre_bytes, hipMemcpyHostToDevice, ctx->stream));
     mcclx::TableArgs t;
     t.segs = static_cast<const mcclx::SegArgs*>(sl.dev);
@@ -439,6 +442,10 @@ int make_ctx(int device, hipStream_t borrowed, bool borrow, mcclx_ctx** out) {
     if (const char* v = getenv("MCCLX_BLOCKS_PER_CU")) {
         int x = atoi(v);
         if (x >= 1 && x <= 16384) ctx->max_blocks = (uint32_t)ctx->cus * (uint32_t)x;
+    }
+    if (const char* v = getenv("MCCLX_FEW_SEGS")) {  // tuning: 0 sends every launch through the table kernel
+        int x = atoi(v);
+        if (x >= 0 && x <= mcclx::kFewSegs) ctx->few_max = (uint32_t)x;
     }
     if (const char* v = getenv("MCCLX_VALIDATE")) ctx->validate = (v[0] == '1');
     if (borrow) {
