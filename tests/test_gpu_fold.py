@@ -161,10 +161,10 @@ def test_fold_f32_accumulate_mode_is_labelled_variant(K, U, k):
         assert not np.array_equal(want, oracle_fold(ins, BF16))
 
 
-@pytest.mark.parametrize("nseg", [2, 8, 9, 100])
+@pytest.mark.parametrize("nseg", [2, 8, 9, 32, 33, 100])
 @pytest.mark.parametrize("dtype", [F32, BF16])
 def test_fold_batched_ragged_segments(K, U, nseg, dtype):
-    """By-value launch (<= 8 segments) and descriptor-table launch (> 8), with
+    """By-value launch (<= 32 segments) and descriptor-table launch (> 32), with
     empty, tiny, tail-only and misaligned segments."""
     rng = np.random.default_rng(nseg)
     k = 3
@@ -276,7 +276,7 @@ def test_many_table_launches_in_flight(K, U):
     rng = np.random.default_rng(99)
     q = K._q(None)
     n = 3001
-    nseg_list = [9, 12, 40, 9, 300, 17, 1000, 10, 64, 9, 2000, 33]
+    nseg_list = [33, 36, 40, 33, 300, 47, 1000, 34, 64, 33, 2000, 35]
     total = max(nseg_list) * n
     a = U.rand_values(rng, total, F32); b = U.rand_values(rng, total, F32)
     da, db = U.to_dev(a, F32), U.to_dev(b, F32)

@@ -1,5 +1,5 @@
 """Randomised parity of mcclx_fold_batched against the oracle: random plans (dtype, io
-mode, k, topology, op, scale constant), 1..40 segments per launch with random lengths
+mode, k, topology, op, scale constant), 1..70 segments per launch with random lengths
 (empty ones included) and element-granular offsets of every stream, outputs checked
 bit for bit including the untouched bytes around every segment.  MCCLX_FUZZ_ROUNDS
 raises the number of launches (default 60, a few seconds)."""
@@ -75,7 +75,7 @@ def test_random_plans_segments_and_offsets(K, U):
     GUARD = 70   # elements kept free on both sides of every stream's range
     for rnd in range(ROUNDS):
         dtype, io, k, binomial, op, scale, mode = random_plan(rng, L)
-        nseg = int(rng.choice([1, 2, 3, 8, 9, 17, 40]))
+        nseg = int(rng.choice([1, 2, 3, 8, 9, 17, 32, 33, 40, 70]))
         big = rnd % 10 == 0
         counts = [int(c) for c in rng.choice([0, 1, 3, 63, 64, 65, 511, 2047, 2048, 2049, 8191, 30011,
                                               262147 if big else 4099], size=nseg)]
