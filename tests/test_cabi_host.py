@@ -4,6 +4,7 @@ workspace sizing, argument checking) matches the oracle.  No compute calls."""
 import ctypes as C
 import os
 import re
+import sys
 
 import numpy as np
 import pytest
@@ -137,3 +138,19 @@ def test_only_one_hip_runtime_is_loaded_whatever_the_import_order():
     assert out.returncode == 0, out.stderr[-2000:]
     libs = [l for l in out.stdout.strip().splitlines() if l]
     assert len(libs) == 1, libs
+
+
+def test_header_is_strict_c99_and_a_plain_c_client_links_and_runs():
+    """include/mcclx.h compiles as C99 with -pedantic -Werror; a C program linked against
+    libmcclx.so uses the host-only entry points (tests/native/cabi_host.c).  The GPU client
+    is compiled here too, so that it travels with the tree."""
+    import subprocess
+    sys.path.insert(0, os.path.join(os.path.dirname(__file__), "native"))
+    import build_native
+    try:
+        exe = build_native.build("cabi_host", force=True)
+        build_native.build("cabi_gpu", force=True)
+    except subprocess.CalledProcessError as e:
+        raise AssertionError(e.stderr)
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0 and r.stdout.strip() == "ok", r.stderr
