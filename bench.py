@@ -307,6 +307,18 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
             rep(i)
         ms = q.timer_end()
         out[f"c2_allreduce_{name}_us_per_bucket"] = round(ms / steps * 1e3, 1)
+    # the fused schedule again, its launches recorded into a graph (no host launch cost between them)
+    import ctypes as C
+    reps = []
+    for s in range(sets):
+        r = L.Replay()
+        r.world, r.algo, r.op, r.dtype = world, L.ALGO_BUTTERFLY, L.AVG, L.F32
+        r.wire_bf16, r.mode, r.acc, r.reserved, r.numel = 1, L.REPLAY_FUSED, L.ACC_STEP, 0, numel
+        ptrs = (C.c_void_p * world)(*[t.data_ptr() for t in tensors[s]])
+        r.tensors, r.workspace, r.workspace_bytes = ptrs, ws.ptr, ws.nbytes
+        reps.append((r, ptrs))
+    ms, _ = measure(lambda i: L.check(L.lib().mcclx_allreduce_replay(q.handle, C.byref(reps[i % sets][0]))), steps, warm)
+    out["c2_allreduce_fused_in_graph_us_per_bucket"] = round(ms / steps * 1e3, 1)
     ws.free()
 
     # C1: ring, 2 ranks, 1 Mi fp32, SUM: one k=2 fold per chunk
