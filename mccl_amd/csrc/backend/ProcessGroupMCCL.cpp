@@ -204,6 +204,7 @@ void ProcessGroupMCCL::flush_engine_() {
         done = true;
         cv.notify_all();
     });
+    BlockingRegion unlocked;
     std::unique_lock<std::mutex> lk(mu);
     cv.wait(lk, [&] { return done; });
 }
@@ -225,11 +226,13 @@ c10::intrusive_ptr<c10d::Work> async_submit_(Progress& engine, mcclx_ctx* ctx, v
         return work;
     }
     work->setSyncCallback([ctx] { check_rc(mcclx_queue_drain(ctx)); });
-    engine.submit([work, body = std::move(body)]() {
+    engine.submit([work, body = std::move(body)]() mutable {
         try {
             body();
+            body = nullptr;  // release the captured tensors before anyone is told the work is done
             work->finish();
         } catch (...) {
+            body = nullptr;
             work->finishWithException(std::current_exception());
         }
     });

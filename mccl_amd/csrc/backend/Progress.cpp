@@ -4,6 +4,23 @@
 
 namespace mccl {
 
+namespace {
+BlockingHooks g_hooks;
+}
+
+void set_blocking_hooks(BlockingHooks hooks) { g_hooks = hooks; }
+
+BlockingRegion::BlockingRegion() {
+    if (g_hooks.enter && g_hooks.leave) {
+        token_ = g_hooks.enter();
+        entered_ = true;
+    }
+}
+
+BlockingRegion::~BlockingRegion() {
+    if (entered_) g_hooks.leave(token_);
+}
+
 Progress::Progress() { thread_ = std::thread([this] { worker(); }); }
 
 Progress::~Progress() { shutdown(); }
@@ -24,7 +41,10 @@ void Progress::shutdown() {
         closing_ = true;
     }
     wake_.notify_all();
-    if (thread_.joinable()) thread_.join();
+    if (thread_.joinable()) {
+        BlockingRegion unlocked;  // the last task may need the caller's interpreter lock to end
+        thread_.join();
+    }
 }
 
 size_t Progress::completed() const {
@@ -45,6 +65,7 @@ void Progress::worker() {
         } catch (...) {
             // the task reports its own failure through its Work object
         }
+        task = nullptr;  // its captures die here, outside the queue lock
         lk.lock();
         ++completed_;
     }

@@ -16,6 +16,31 @@
 
 namespace mccl {
 
+// A host with an interpreter lock (CPython's GIL) registers a pair of hooks.
+// They bracket every place where a caller blocks until the worker thread has
+// got somewhere, because a task may need that lock before it can end: when a
+// task drops the last reference to a tensor that Python created, the tensor's
+// destructor takes the GIL.  A caller that joined the worker while holding the
+// GIL (a process group destroyed from Python does) would then wait for ever.
+struct BlockingHooks {
+    void* (*enter)() = nullptr;    // give the lock up if this thread holds it; returns a token
+    void (*leave)(void*) = nullptr;  // take it back
+};
+void set_blocking_hooks(BlockingHooks hooks);
+
+// RAII use of the hooks; a no-op when none are registered.
+class BlockingRegion {
+public:
+    BlockingRegion();
+    ~BlockingRegion();
+    BlockingRegion(const BlockingRegion&) = delete;
+    BlockingRegion& operator=(const BlockingRegion&) = delete;
+
+private:
+    void* token_ = nullptr;
+    bool entered_ = false;
+};
+
 class Progress {
 public:
     using Task = std::function<void()>;

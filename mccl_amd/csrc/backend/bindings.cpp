@@ -27,6 +27,16 @@ namespace py = pybind11;
 
 namespace {
 
+// Blocking hooks for the engine (Progress.hpp): give the GIL up while a caller
+// waits for the worker thread, if this thread holds it.
+void* gil_release_if_held() {
+    if (!Py_IsInitialized() || !PyGILState_Check()) return nullptr;
+    return PyEval_SaveThread();
+}
+void gil_take_back(void* token) {
+    if (token) PyEval_RestoreThread(static_cast<PyThreadState*>(token));
+}
+
 // Submits n tasks; task i throws when bit i of throw_mask is set (i < 64).
 // Returns the order in which the non-throwing tasks ran.
 std::vector<int> progress_order(int n, uint64_t throw_mask, bool use_destructor) {
@@ -48,6 +58,20 @@ std::vector<int> progress_order(int n, uint64_t throw_mask, bool use_destructor)
         }
     }
     return order;
+}
+
+// Called WITH the GIL held: a task that needs the GIL (as one that drops the last
+// reference to a Python-created tensor does) must not dead-lock the shutdown.
+int progress_shutdown_while_task_needs_gil() {
+    int ran = 0;
+    mccl::Progress p;
+    p.submit([&ran] {
+        std::this_thread::sleep_for(std::chrono::milliseconds(20));
+        py::gil_scoped_acquire gil;
+        ran = 1;
+    });
+    p.shutdown();
+    return ran;
 }
 
 // Microseconds a submit() takes while the worker is busy with a 50 ms task.
@@ -134,6 +158,7 @@ std::vector<std::string> mesh_probe(int world, int rounds, int absent, int timeo
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.doc() = "mccl_amd native backend: c10d ProcessGroup over libmcclx";
     py::register_exception<mccl::MCCLError>(m, "MCCLError", PyExc_RuntimeError);
+    mccl::set_blocking_hooks({&gil_release_if_held, &gil_take_back});
 
     m.def("_create_process_group_mccl",
           [](const c10::intrusive_ptr<c10d::Store>& store, int rank, int size,
@@ -154,6 +179,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
 
     m.def("_test_progress_order", &progress_order, py::arg("n"), py::arg("throw_mask") = 0,
           py::arg("use_destructor") = false, py::call_guard<py::gil_scoped_release>());
+    m.def("_test_progress_shutdown_while_task_needs_gil", &progress_shutdown_while_task_needs_gil);
     m.def("_test_progress_submit_latency_us", &progress_submit_latency_us,
           py::call_guard<py::gil_scoped_release>());
     m.def("_test_work", &work_probe, py::arg("mode"), py::arg("wait_ms") = 1000,

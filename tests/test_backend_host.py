@@ -93,3 +93,17 @@ def test_factory_fails_loudly_without_a_gpu(CX):
         CX._create_process_group_mccl(dist.HashStore(), 0, 1, datetime.timedelta(seconds=5))
     with pytest.raises(RuntimeError, match="rank/size invalid"):
         CX._create_process_group_mccl(dist.HashStore(), 3, 2, datetime.timedelta(seconds=5))
+
+
+def test_engine_shutdown_under_the_gil_does_not_deadlock_with_a_task_that_needs_it(CX):
+    """A process group dropped from Python is destroyed with the GIL held and joins its engine
+    thread; the engine's last task may be releasing a tensor Python created, which takes the GIL.
+    The join therefore gives the GIL up (regression: rank threads froze when groups were
+    created and dropped in a loop)."""
+    import threading
+    res = []
+    t = threading.Thread(target=lambda: res.append(CX._test_progress_shutdown_while_task_needs_gil()), daemon=True)
+    t.start()
+    t.join(20)
+    assert not t.is_alive(), "shutdown dead-locked against a task waiting for the GIL"
+    assert res == [1]
