@@ -3,12 +3,14 @@
 #include <c10/hip/HIPFunctions.h>
 #include <c10/hip/HIPStream.h>
 
+#include <algorithm>
 #include <condition_variable>
 #include <cstdlib>
 #include <cstring>
 #include <functional>
 #include <map>
 #include <mutex>
+#include <tuple>
 
 #include "backend/Errors.hpp"
 #include "backend/LocalMesh.hpp"
@@ -88,19 +90,101 @@ struct ProcessGroupMCCL::Shared {
     at::Tensor scratch;
     int device = 0;
 
+    // Recorded allreduces.  A DDP bucket is reduced again and again at the same
+    // addresses; from its second occurrence on, the launches of one allreduce
+    // (encode, fold, decode/copy legs) are recorded into a HIP graph and replayed
+    // with one submission, which removes the host's launch gaps between them.
+    // The key is everything the launches depend on; MCCL_GRAPH_CACHE=0 turns it off.
+    struct GraphKey {
+        int world, algo, op, dtype, wire;
+        uint64_t numel;
+        void* workspace;
+        std::vector<void*> tensors;
+        bool operator<(const GraphKey& o) const {
+            return std::tie(world, algo, op, dtype, wire, numel, workspace, tensors) <
+                   std::tie(o.world, o.algo, o.op, o.dtype, o.wire, o.numel, o.workspace, o.tensors);
+        }
+    };
+    struct GraphEntry {
+        mcclx_graph* graph = nullptr;
+        uint64_t seen = 0, last_use = 0;
+    };
+    static constexpr size_t kMaxGraphs = 256;
+    std::map<GraphKey, GraphEntry> graphs;
+    uint64_t use_clock = 0;
+    uint64_t graph_hits = 0;
+    bool graphs_enabled = true;
+
+    Shared() {
+        const char* e = std::getenv("MCCL_GRAPH_CACHE");
+        graphs_enabled = !(e && e[0] == '0');
+    }
     ~Shared() {
+        drop_graphs();
         if (ctx) mcclx_destroy(ctx);
+    }
+    void drop_graphs() {
+        for (auto& kv : graphs)
+            if (kv.second.graph) (void)mcclx_graph_destroy(ctx, kv.second.graph);
+        graphs.clear();
     }
     void* workspace(uint64_t nbytes) {
         if (nbytes == 0) return nullptr;
         if (!scratch.defined() || static_cast<uint64_t>(scratch.numel()) < nbytes + 256) {
             check_rc(mcclx_queue_drain(ctx));  // nothing may still read the old buffer
+            drop_graphs();                     // recorded launches point into it
             scratch = at::empty({static_cast<int64_t>(nbytes + 256)},
                                 at::TensorOptions().dtype(at::kByte).device(at::kCUDA, device));
             order_after_allocator(ctx, device);
         }
         auto p = reinterpret_cast<uintptr_t>(scratch.data_ptr());
         return reinterpret_cast<void*>((p + 255) / 256 * 256);
+    }
+
+    // One allreduce of the group: replayed from its graph when there is one,
+    // recorded on its second occurrence, issued launch by launch otherwise.
+    void allreduce(const mcclx_replay& rp) {
+        if (!graphs_enabled) {
+            check_rc(mcclx_allreduce_replay(ctx, &rp));
+            return;
+        }
+        GraphKey key{rp.world, rp.algo, rp.op, rp.dtype, rp.wire_bf16, rp.numel, rp.workspace,
+                     std::vector<void*>(rp.tensors, rp.tensors + rp.world)};
+        GraphEntry& e = graphs[key];
+        e.last_use = ++use_clock;
+        ++e.seen;
+        if (!e.graph && e.seen >= 2) {
+            check_rc(mcclx_graph_begin(ctx));
+            int rc = mcclx_allreduce_replay(ctx, &rp);
+            std::string why = rc == MCCLX_OK ? "" : mcclx_last_error();
+            mcclx_graph* g = nullptr;
+            int rc_end = mcclx_graph_end(ctx, &g);
+            if (rc != MCCLX_OK) {
+                if (g) (void)mcclx_graph_destroy(ctx, g);
+                throw KernelError(why);
+            }
+            check_rc(rc_end);
+            e.graph = g;
+        }
+        if (e.graph) {
+            check_rc(mcclx_graph_launch(ctx, e.graph));
+            ++graph_hits;
+        } else {
+            check_rc(mcclx_allreduce_replay(ctx, &rp));
+        }
+        if (graphs.size() > kMaxGraphs) evict();
+    }
+    void evict() {  // drop the least recently used half
+        std::vector<std::pair<uint64_t, const GraphKey*>> order;
+        for (auto& kv : graphs) order.emplace_back(kv.second.last_use, &kv.first);
+        std::sort(order.begin(), order.end());
+        std::vector<GraphKey> victims;
+        for (size_t i = 0; i < order.size() / 2; ++i) victims.push_back(*order[i].second);
+        for (auto& k : victims) {
+            auto it = graphs.find(k);
+            if (it->second.graph) (void)mcclx_graph_destroy(ctx, it->second.graph);
+            graphs.erase(it);
+        }
     }
 };
 
@@ -163,6 +247,8 @@ ProcessGroupMCCL::~ProcessGroupMCCL() {
     shared_.reset();
     if (!mesh_key_.empty()) LocalMesh::forget(mesh_key_);
 }
+
+uint64_t ProcessGroupMCCL::graphHits() const { return shared_ ? shared_->graph_hits : 0; }
 
 void* ProcessGroupMCCL::my_stream() const {
     return static_cast<void*>(c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(device_)).stream());
@@ -318,7 +404,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
             uint64_t need = std::max(mcclx_replay_workspace_bytes(&rp), mcclx_replay_workspace_bytes(&st));
             rp.workspace = shared->workspace(need);
             rp.workspace_bytes = need;
-            check_rc(mcclx_allreduce_replay(ctx, &rp));
+            shared->allreduce(rp);
         }
         check_rc(mcclx_queue_drain(ctx));  // mccl_queue_drain, :178
     });

@@ -71,6 +71,8 @@ public:
 
     // Algorithm the last allreduce on this rank ran (MCCLX_ALGO_*), for tests.
     int lastAlgo() const { return last_algo_; }
+    // Allreduces of this rank's group that were replayed from a recorded graph, for tests.
+    uint64_t graphHits() const;
 
 private:
     struct Shared;  // reduce queue + scratch shared by the ranks of one mesh

@@ -176,6 +176,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         auto* p = dynamic_cast<mccl::ProcessGroupMCCL*>(pg.get());
         return p ? p->lastAlgo() : -1;
     });
+    m.def("_graph_hits", [](const c10::intrusive_ptr<c10d::Backend>& pg) {
+        auto* p = dynamic_cast<mccl::ProcessGroupMCCL*>(pg.get());
+        return p ? p->graphHits() : uint64_t(0);
+    });
 
     m.def("_test_progress_order", &progress_order, py::arg("n"), py::arg("throw_mask") = 0,
           py::arg("use_destructor") = false, py::call_guard<py::gil_scoped_release>());

@@ -498,3 +498,66 @@ def test_recv_times_out_when_nothing_was_sent(CX):
     assert not any(t.is_alive() for t in ts)
     assert "Timeout" in msgs[0] and "nothing arrived from rank 1" in msgs[0]
     assert msgs[2] == [9.0] * 4
+
+
+# ---- recorded allreduces ---------------------------------------------------------------
+
+@pytest.mark.parametrize("wire", [False, True])
+def test_repeated_allreduce_is_replayed_from_a_graph_and_stays_bit_exact(CX, U, monkeypatch, wire):
+    """The same buffers reduced again and again (a DDP bucket): from the second time on the
+    launches are recorded, later calls replay the graph.  Every call is checked against the
+    oracle, with other work on torch's stream and other collectives between the replays."""
+    world, n = 3, 300_007
+    monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "butterfly")
+    if wire:
+        monkeypatch.setenv("MCCL_WIRE_DTYPE", "bf16")
+    else:
+        monkeypatch.delenv("MCCL_WIRE_DTYPE", raising=False)
+    monkeypatch.delenv("MCCL_GRAPH_CACHE", raising=False)
+    rng = np.random.default_rng(77)
+    rounds = 8
+    data = [[U.rand_values(rng, n, F32, scale=1e-2, specials=(i == 3)) for _ in range(world)] for i in range(rounds)]
+
+    def fn(r, pg):
+        bucket = torch.empty(n, device="cuda")          # one address for every round
+        other = torch.empty(1000, device="cuda")
+        got = []
+        for i in range(rounds):
+            bucket.copy_(torch.from_numpy(data[i][r]))
+            o = dist.AllreduceOptions(); o.reduceOp = dist.ReduceOp.AVG
+            pg.allreduce([bucket], o).wait()
+            got.append(U.bits(bucket).copy())
+            other.fill_(float(i)).mul_(2.0)                # unrelated eager work between replays
+            if i % 3 == 1:
+                pg.broadcast([other], dist.BroadcastOptions()).wait()
+        return got, CX._graph_hits(pg)
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for i in range(rounds):
+        want = [x.copy() for x in data[i]]
+        rc, used = orc.pg_allreduce(want, F32, AVG, wire_bf16=wire, env_algo="butterfly", threads=4)
+        assert rc == 0 and used == BUTTERFLY
+        for r in range(world):
+            w = want[r].view(np.uint32)
+            g = out[r][0][i]
+            same = (g == w) | (np.isnan(g.view(np.float32)) & np.isnan(w.view(np.float32)))
+            assert same.all(), (i, r, int((~same).sum()))
+    assert out[0][1] >= rounds - 2          # first call eager, second records and replays
+
+
+def test_graph_cache_can_be_switched_off(CX, monkeypatch):
+    monkeypatch.setenv("MCCL_GRAPH_CACHE", "0")
+    monkeypatch.delenv("MCCL_WIRE_DTYPE", raising=False)
+
+    def fn(r, pg):
+        t = torch.empty(4096, device="cuda")
+        for i in range(5):
+            t.fill_(float(r + i))
+            pg.allreduce([t]).wait()
+            assert float(t[0]) == 2.0 * i + 1.0
+        return CX._graph_hits(pg)
+
+    out, errs = run_ranks(CX, 2, fn)
+    assert errs == [None, None], errs
+    assert out == [0, 0]
