@@ -14,6 +14,7 @@
 
 #include "backend/Errors.hpp"
 #include "backend/LocalMesh.hpp"
+#include "backend/Logging.hpp"
 #include "backend/Progress.hpp"
 #include "backend/WorkMCCL.hpp"
 
@@ -165,6 +166,8 @@ struct ProcessGroupMCCL::Shared {
             }
             check_rc(rc_end);
             e.graph = g;
+            MCCL_DEBUG("allreduce recorded: world %d algo %d op %d dtype %d wire %d numel %llu (%zu graphs kept)",
+                       rp.world, rp.algo, rp.op, rp.dtype, rp.wire_bf16, (unsigned long long)rp.numel, graphs.size());
         }
         if (e.graph) {
             check_rc(mcclx_graph_launch(ctx, e.graph));
@@ -239,6 +242,8 @@ ProcessGroupMCCL::ProcessGroupMCCL(c10::intrusive_ptr<c10d::Store> store, int ra
     }
     ctx_ = shared_->ctx;
     engine_ = std::make_unique<Progress>();
+    MCCL_INFO("rank %d of %d joined in-process mesh %s on GPU %d (%d CUs)", rank, size, mesh_key_.c_str(), device_,
+              mcclx_device_cus(ctx_));
 }
 
 ProcessGroupMCCL::~ProcessGroupMCCL() {
@@ -312,13 +317,20 @@ c10::intrusive_ptr<c10d::Work> async_submit_(Progress& engine, mcclx_ctx* ctx, v
         return work;
     }
     work->setSyncCallback([ctx] { check_rc(mcclx_queue_drain(ctx)); });
-    engine.submit([work, body = std::move(body)]() mutable {
+    engine.submit([work, title, body = std::move(body)]() mutable {
         try {
             body();
             body = nullptr;  // release the captured tensors before anyone is told the work is done
             work->finish();
         } catch (...) {
             body = nullptr;
+            try {
+                throw;
+            } catch (const std::exception& e) {
+                MCCL_ERROR("%s failed: %s", title, e.what());
+            } catch (...) {
+                MCCL_ERROR("%s failed with a non-standard exception", title);
+            }
             work->finishWithException(std::current_exception());
         }
     });
@@ -364,6 +376,8 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
         c.algo.push_back(mcclx_select_algo(env_alg, tree_below, bytes, t.numel(), world));  // :134-145
     }
     last_algo_ = c.algo.back();
+    MCCL_DEBUG("rank %d allreduce: %zu tensor(s), first numel %llu, op %d, algo %d, wire %s", getRank(), tensors.size(),
+               (unsigned long long)c.numel[0], op, last_algo_, wire ? "bf16" : "native");
     flush_engine_();
 
     auto shared = shared_;

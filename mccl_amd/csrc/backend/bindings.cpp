@@ -19,6 +19,7 @@
 
 #include "backend/Errors.hpp"
 #include "backend/LocalMesh.hpp"
+#include "backend/Logging.hpp"
 #include "backend/ProcessGroupMCCL.hpp"
 #include "backend/Progress.hpp"
 #include "backend/WorkMCCL.hpp"
@@ -183,6 +184,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
 
     m.def("_test_progress_order", &progress_order, py::arg("n"), py::arg("throw_mask") = 0,
           py::arg("use_destructor") = false, py::call_guard<py::gil_scoped_release>());
+    m.def("_test_log", [](int level, const std::string& text) {
+        mccl::log::emit(level, "bindings.cpp", 0, "%s", text.c_str());
+        return mccl::log::enabled(level);
+    });
     m.def("_test_progress_shutdown_while_task_needs_gil", &progress_shutdown_while_task_needs_gil);
     m.def("_test_progress_submit_latency_us", &progress_submit_latency_us,
           py::call_guard<py::gil_scoped_release>());

@@ -4,6 +4,7 @@ reference's own engine from oracle/_ref run on the same cases), the Work
 object (csrc/backend/WorkMCCL.cpp), the in-process mesh, registration."""
 import ctypes as C
 import datetime
+import os
 
 import pytest
 
@@ -107,3 +108,27 @@ def test_engine_shutdown_under_the_gil_does_not_deadlock_with_a_task_that_needs_
     t.join(20)
     assert not t.is_alive(), "shutdown dead-locked against a task waiting for the GIL"
     assert res == [1]
+
+
+def test_logger_levels_and_line_format():
+    """DISTRO_LOG_LEVEL as in the reference (csrc/common/Logging.hpp:22-78): default WARN, names in
+    any case or digits, lines '[MCCL LEVEL epoch-ms file:line] text' on stderr."""
+    import re
+    import subprocess
+    import sys
+    code = ("import mccl_amd; from mccl_amd import _C; "
+            "print([int(_C._test_log(l, 'message %d' % l)) for l in range(7)])")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for setting, first in ((None, 3), ("debug", 1), ("TRACE", 0), ("4", 4), ("off", 7), ("nonsense", 3)):
+        env = dict(os.environ)
+        env.pop("DISTRO_LOG_LEVEL", None)
+        if setting is not None:
+            env["DISTRO_LOG_LEVEL"] = setting
+        r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=root, env=env, timeout=120)
+        assert r.returncode == 0, r.stderr
+        enabled = eval(r.stdout.strip().splitlines()[-1])
+        assert enabled == [int(first <= l < 6) for l in range(7)], (setting, enabled)
+        lines = [l for l in r.stderr.splitlines() if l.startswith("[MCCL ")]
+        assert len(lines) == sum(enabled)
+        for l in lines:
+            assert re.fullmatch(r"\[MCCL (TRACE|DEBUG|INFO |WARN |ERROR|FATAL) \d{13} bindings\.cpp:0\] message \d", l), l
