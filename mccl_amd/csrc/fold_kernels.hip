@@ -53,6 +53,9 @@ namespace {
 #ifndef MCCLX_TUNE_HWCVT
 #define MCCLX_TUNE_HWCVT 1  // 1: v_cvt_pk_bf16_f32 + NaN fix-up; 0: integer rounding
 #endif
+#ifndef MCCLX_TUNE_XCD
+#define MCCLX_TUNE_XCD 0    // N > 0: give each of N XCDs one contiguous N-th of a segment's tiles
+#endif
 #ifndef MCCLX_TUNE_PEEL
 #define MCCLX_TUNE_PEEL 1   // scalar head peel up to the output's 128-byte boundary
 #endif
@@ -423,8 +426,15 @@ template <class C>
 __global__ void __launch_bounds__(kBlock) fold_few_kernel(FewArgs a) {
     const SegArgs& s = a.seg[blockIdx.y];
     const uint64_t span = (uint64_t)C::U * kBlock;
+#if MCCLX_TUNE_XCD
+    // workgroups go to the XCDs round robin: block b runs on XCD b % N
+    const uint32_t per = gridDim.x / MCCLX_TUNE_XCD;  // the grid is a multiple of N
+    const uint32_t tile = (blockIdx.x % MCCLX_TUNE_XCD) * per + blockIdx.x / MCCLX_TUNE_XCD;
+    fold_segment<C>(s, a.scale, a.has_scale != 0, (uint64_t)tile * span, ~0ull >> 1, tile == 0);
+#else
     fold_segment<C>(s, a.scale, a.has_scale != 0, (uint64_t)blockIdx.x * span,
                     (uint64_t)gridDim.x * span, blockIdx.x == 0);
+#endif
 }
 
 // A value that is the same in every lane, moved to scalar registers.  The
@@ -498,6 +508,9 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
         uint64_t cap = lp.max_blocks / (uint32_t)a.nseg;
         if (cap < 1) cap = 1;
         if (gx > cap) gx = cap;
+#if MCCLX_TUNE_XCD
+        gx = (gx + MCCLX_TUNE_XCD - 1) / MCCLX_TUNE_XCD * MCCLX_TUNE_XCD;
+#endif
         fold_few_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(kBlock), 0, st>>>(a);
     }
     return hipGetLastError();
