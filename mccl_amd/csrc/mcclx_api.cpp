@@ -325,7 +325,20 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
 
     mcclx::LaunchParams lp;
     lp.max_blocks = ctx->max_blocks;
-    if (nseg <= ctx->few_max) {
+    // By value: the grid is (tiles of the longest segment) x (segments), so a launch
+    // whose segments differ wildly in length would consist mostly of blocks with
+    // nothing to do; such a launch takes the table, which has one block per tile.
+    bool by_value = nseg <= ctx->few_max;
+    if (by_value && nseg > 4) {
+        uint64_t longest = 0, total = 0;
+        for (uint32_t s = 0; s < nseg; ++s) {
+            uint64_t n = mcclx::items_for(key, segs[s].count);
+            total += n;
+            if (n > longest) longest = n;
+        }
+        by_value = longest * nseg <= 4 * total + 64;
+    }
+    if (by_value) {
         mcclx::FewArgs a;
         memset(&a, 0, sizeof a);
         for (uint32_t s = 0; s < nseg; ++s) memcpy(&a.seg[s], &segs[s], sizeof(mcclx_seg));

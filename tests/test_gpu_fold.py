@@ -323,3 +323,26 @@ def test_two_queues_from_two_threads(K, U):
         for _ in range(20):
             orc.reduce(want, data[i][1], BF16, SUM, threads=4)
         assert np.array_equal(res[i], want)
+
+
+def test_one_long_segment_among_many_short_ones(K, U):
+    """A launch of 9..32 segments travels by value unless its segments differ so much in
+    length that most of the (longest x segments) grid would idle; either way the result
+    is the same."""
+    rng = np.random.default_rng(31)
+    for nseg, long_n in ((12, 3_000_001), (32, 1_000_003), (6, 2_000_003)):
+        counts = [long_n] + [int(c) for c in rng.integers(1, 300, nseg - 1)]
+        total = sum(counts) + 16 * nseg
+        a = U.rand_values(rng, total, BF16, scale=1e-2); b = U.rand_values(rng, total, BF16, scale=1e-2)
+        da, db = U.to_dev(a, BF16), U.to_dev(b, BF16)
+        out = torch.zeros(total, dtype=torch.bfloat16, device="cuda")
+        want = np.zeros(total, np.uint16)
+        segs, off = [], 0
+        for n in counts:
+            segs.append(K.make_seg(out.data_ptr() + 2 * off, 0, [da.data_ptr() + 2 * off, db.data_ptr() + 2 * off], n))
+            x = a[off:off + n].copy(); orc.reduce(x, b[off:off + n].copy(), BF16, SUM)
+            want[off:off + n] = x
+            off += n + 16
+        K._q(None).fold(K.make_plan(BF16, 2), segs)
+        K.hip_sync()
+        assert np.array_equal(U.bits(out), want), (nseg, long_n)
