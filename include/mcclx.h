@@ -171,6 +171,19 @@ MCCLX_API int mcclx_fold_batched(mcclx_ctx* ctx, const mcclx_plan* plan, const m
  * ProcessGroupMCCL.cpp:232-273). */
 MCCLX_API int mcclx_copy(mcclx_ctx* ctx, void* dst, const void* src, uint64_t nbytes);
 
+/* Many copies with one launch: the allgather leg of a schedule hands every
+ * reduced chunk to every other rank (AllreduceAlgos.cpp:77-86, 185-200; the
+ * tree's broadcast :119-126), N-1 sends per chunk in the reference.  Ranges of
+ * different descriptors must not overlap each other's destinations; a
+ * descriptor with nbytes == 0 or dst == src is skipped.  A few large copies are
+ * issued one launch each (that streams best); many small ones go out together. */
+typedef struct mcclx_copy_desc {
+    void* dst;
+    const void* src;
+    uint64_t nbytes;
+} mcclx_copy_desc;
+MCCLX_API int mcclx_copy_batched(mcclx_ctx* ctx, const mcclx_copy_desc* descs, uint32_t n);
+
 /* ---- reduce queue: completion and cross-stream ordering --------------------- */
 
 /* Block until every launch on the queue has finished.  Replaces
@@ -276,6 +289,14 @@ MCCLX_API uint64_t mcclx_replay_workspace_bytes(const mcclx_replay* r);
  * on this GPU: every send/recv becomes a device copy (STEPWISE) or a direct
  * read of the peer's chunk (FUSED).  Both modes produce bit-identical tensors. */
 MCCLX_API int mcclx_allreduce_replay(mcclx_ctx* ctx, const mcclx_replay* r);
+
+/* The same for a list of tensors, as ProcessGroupMCCL::allreduce takes one
+ * (ProcessGroupMCCL.cpp:122-168 runs the list one tensor after another).  Here
+ * consecutive entries that share world, algorithm, op, dtype and wire setting
+ * are issued together: one launch per phase (encode, fold, cast, copies) for
+ * the whole run instead of one per tensor -- thousands of small tree messages
+ * become a handful of launches.  Results are those of n single replays. */
+MCCLX_API int mcclx_allreduce_replay_many(mcclx_ctx* ctx, const mcclx_replay* replays, uint32_t n);
 
 /* _reduce_scatter_base (ProcessGroupMCCL.cpp:331-390): ins[r] holds
  * world*chunk_numel elements, outs[r] receives chunk_numel.  FUSED: one

@@ -31,6 +31,10 @@ class Seg(C.Structure):
                 ("inp", C.c_void_p * MAX_INPUTS), ("count", C.c_uint64)]
 
 
+class CopyDesc(C.Structure):
+    _fields_ = [("dst", C.c_void_p), ("src", C.c_void_p), ("nbytes", C.c_uint64)]
+
+
 class Plan(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("io", C.c_int32), ("k", C.c_int32), ("topo", C.c_int32),
                 ("op", C.c_int32), ("acc", C.c_int32), ("scale_mode", C.c_int32),
@@ -70,6 +74,7 @@ SIGNATURES = {
     "mcclx_fold": (_i, [_vp, C.POINTER(Plan), C.POINTER(Seg)]),
     "mcclx_fold_batched": (_i, [_vp, C.POINTER(Plan), C.POINTER(Seg), C.c_uint32]),
     "mcclx_copy": (_i, [_vp, _vp, _vp, _u64]),
+    "mcclx_copy_batched": (_i, [_vp, C.POINTER(CopyDesc), C.c_uint32]),
     "mcclx_queue_drain": (_i, [_vp]),
     "mcclx_queue_wait_stream": (_i, [_vp, _vp]),
     "mcclx_stream_wait_queue": (_i, [_vp, _vp]),
@@ -90,6 +95,7 @@ SIGNATURES = {
     "mcclx_select_algo": (_i, [C.c_char_p, _i64, _u64, _i64, _i]),
     "mcclx_replay_workspace_bytes": (_u64, [C.POINTER(Replay)]),
     "mcclx_allreduce_replay": (_i, [_vp, C.POINTER(Replay)]),
+    "mcclx_allreduce_replay_many": (_i, [_vp, C.POINTER(Replay), C.c_uint32]),
     "mcclx_reduce_scatter_replay": (_i, [_vp, _i, _pp, _pp, _i, _u64, _i, _i, _i]),
     "mcclx_reduce_scatter_shares": (_i, [_vp, _i, _pp, _pp, _i, _u64, _i, _i, _i]),
     "mcclx_allgather_replay": (_i, [_vp, _i, _pp, _pp, _u64]),

@@ -392,16 +392,22 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
                        "allreduce: ranks disagree on the reduce op or MCCL_WIRE_DTYPE");
             check_rc(mcclx_queue_wait_stream(ctx, all[r].stream));  // mps_stream_sync, :172
         }
+        // one replay per tensor of the list; the reference runs them one after another
+        // (ProcessGroupMCCL.cpp:122-168), here a list is issued together so that
+        // entries sharing a plan need one launch per phase for all of them
+        std::vector<std::vector<void*>> ptrs(nt, std::vector<void*>(static_cast<size_t>(world)));
+        std::vector<mcclx_replay> reps(nt);
+        std::vector<uint64_t> need(nt), offset(nt);
+        uint64_t total = 0;
         for (size_t i = 0; i < nt; ++i) {
-            std::vector<void*> ptrs(static_cast<size_t>(world));
             for (int r = 0; r < world; ++r) {
                 MCCL_CHECK(all[r].numel[i] == all[0].numel[i] && all[r].dtype[i] == all[0].dtype[i],
                            "allreduce: ranks passed tensors of different size or dtype");
                 MCCL_CHECK(all[r].algo[i] == all[0].algo[i],
                            "allreduce: ranks resolved different algorithms (MCCL_ALLREDUCE_ALGO / MCCL_TREE_BELOW differ)");
-                ptrs[static_cast<size_t>(r)] = all[r].dst[i];
+                ptrs[i][static_cast<size_t>(r)] = all[r].dst[i];
             }
-            mcclx_replay rp;
+            mcclx_replay& rp = reps[i];
             std::memset(&rp, 0, sizeof rp);
             rp.world = world;
             rp.algo = all[0].algo[i];
@@ -411,15 +417,23 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
             rp.mode = MCCLX_REPLAY_FUSED;
             rp.acc = MCCLX_ACC_STEP;
             rp.numel = all[0].numel[i];
-            rp.tensors = ptrs.data();
+            rp.tensors = ptrs[i].data();
             // size for the stepwise fallback too (binary-only ops, wide worlds)
             mcclx_replay st = rp;
             st.mode = MCCLX_REPLAY_STEPWISE;
-            uint64_t need = std::max(mcclx_replay_workspace_bytes(&rp), mcclx_replay_workspace_bytes(&st));
-            rp.workspace = shared->workspace(need);
-            rp.workspace_bytes = need;
-            shared->allreduce(rp);
+            need[i] = (std::max(mcclx_replay_workspace_bytes(&rp), mcclx_replay_workspace_bytes(&st)) + 255) / 256 * 256;
+            offset[i] = total;
+            total += need[i];
         }
+        char* ws = static_cast<char*>(shared->workspace(total));
+        for (size_t i = 0; i < nt; ++i) {
+            reps[i].workspace = need[i] ? ws + offset[i] : nullptr;
+            reps[i].workspace_bytes = need[i];
+        }
+        if (nt == 1)
+            shared->allreduce(reps[0]);  // a single bucket: recorded and replayed when it comes again
+        else
+            check_rc(mcclx_allreduce_replay_many(ctx, reps.data(), static_cast<uint32_t>(nt)));
         check_rc(mcclx_queue_drain(ctx));  // mccl_queue_drain, :178
     });
     return make_completed(c10d::OpType::ALLREDUCE, tensors, "mccl:allreduce");

@@ -61,7 +61,81 @@ __global__ void __launch_bounds__(kBlock) copy_kernel(uint8_t* dst, const uint8_
         if (i < nbytes) gd[i] = gs[i];
     }
 }
+__device__ __forceinline__ uint32_t uni32(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ uint64_t uni64(uint64_t v) {
+    return ((uint64_t)uni32((uint32_t)(v >> 32)) << 32) | uni32((uint32_t)v);
+}
+
+// Many copies, one launch: work item w is tile (w - first_item[c]) of copy c.
+// A tile is kManyU * kBlock packets of 16 bytes (16 KiB); tile 0 also moves the
+// bytes behind the last whole packet.  The loop bound is fixed at launch.
+constexpr int kManyU = 4;
+
+template <int A>
+__global__ void __launch_bounds__(kBlock) copy_many_kernel(CopyTable t) {
+    typedef typename Packet<A>::type V;
+    const uint64_t span = (uint64_t)kManyU * kBlock;
+    for (uint32_t w = blockIdx.x; w < t.total_items; w += gridDim.x) {
+        uint32_t c, tile;
+        if (t.uniform_items) {  // every copy has the same number of tiles: no search
+            c = w / t.uniform_items;
+            tile = w - c * t.uniform_items;
+        } else {
+            uint32_t lo = 0, hi = t.n;  // first_item[lo] <= w < first_item[hi]
+            while (hi - lo > 1) {
+                uint32_t mid = (lo + hi) >> 1;
+                if ((uint32_t)t.first_item[mid] <= w) lo = mid; else hi = mid;
+            }
+            c = lo;
+            tile = w - (uint32_t)t.first_item[c];
+        }
+        c = uni32(c);
+        tile = uni32(tile);
+        const CopyDesc* __restrict__ d = t.descs + c;
+        const MCCLX_GLOBAL uint8_t* gs = (const MCCLX_GLOBAL uint8_t*)uni64(reinterpret_cast<uint64_t>(d->src));
+        MCCLX_GLOBAL uint8_t* gd = (MCCLX_GLOBAL uint8_t*)uni64(reinterpret_cast<uint64_t>(d->dst));
+        const uint64_t nbytes = uni64(d->nbytes);
+        const uint64_t P = nbytes / 16;
+        const uint64_t base = (uint64_t)tile * span;
+        if (base + span <= P) {
+            u32x4 v[kManyU];
+#pragma unroll
+            for (int u = 0; u < kManyU; ++u)
+                v[u] = COPY_LD((const MCCLX_GLOBAL V*)(gs + (base + (uint64_t)u * kBlock + threadIdx.x) * 16));
+#pragma unroll
+            for (int u = 0; u < kManyU; ++u)
+                COPY_ST((MCCLX_GLOBAL V*)(gd + (base + (uint64_t)u * kBlock + threadIdx.x) * 16), v[u]);
+        } else {
+            for (uint64_t p = base + threadIdx.x; p < P; p += kBlock) {
+                u32x4 v = COPY_LD((const MCCLX_GLOBAL V*)(gs + p * 16));
+                COPY_ST((MCCLX_GLOBAL V*)(gd + p * 16), v);
+            }
+        }
+        if (tile == 0) {
+            uint64_t i = P * 16 + threadIdx.x;
+            if (i < nbytes) gd[i] = gs[i];
+        }
+    }
+}
 }  // namespace
+
+uint64_t copy_items(uint64_t nbytes) {
+    const uint64_t span = (uint64_t)kManyU * kBlock * 16;
+    uint64_t n = (nbytes + span - 1) / span;
+    return n ? n : (nbytes ? 1 : 0);
+}
+
+hipError_t launch_copy_many(hipStream_t st, const CopyTable& t, int align, uint32_t max_blocks) {
+    if (t.total_items == 0) return hipSuccess;
+    uint32_t g = t.total_items < max_blocks ? t.total_items : max_blocks;
+    if (align == 4)
+        copy_many_kernel<4><<<dim3(g), dim3(kBlock), 0, st>>>(t);
+    else if (align == 2)
+        copy_many_kernel<2><<<dim3(g), dim3(kBlock), 0, st>>>(t);
+    else
+        copy_many_kernel<1><<<dim3(g), dim3(kBlock), 0, st>>>(t);
+    return hipGetLastError();
+}
 
 hipError_t launch_copy(hipStream_t st, void* dst, const void* src, uint64_t nbytes,
                        uint32_t max_blocks) {

@@ -60,6 +60,25 @@ uint32_t items_for(const PlanKey& key, uint64_t count);
 // hipErrorInvalidValue = no kernel for this plan.
 hipError_t launch_fold(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
 
+// Many copies in one launch: descriptors and nseg+1 work-item prefix sums in
+// device memory (mirrors mcclx_copy_desc).
+struct CopyDesc {
+    void* dst;
+    const void* src;
+    uint64_t nbytes;
+};
+struct CopyTable {
+    const CopyDesc* __restrict__ descs;
+    const uint64_t* __restrict__ first_item;
+    uint32_t total_items;
+    uint32_t uniform_items;  // >0: every copy has this many work items
+    uint32_t n;
+};
+// Work items (tiles) one copy of nbytes splits into.
+uint64_t copy_items(uint64_t nbytes);
+// `align`: the widest of 4 / 2 / 1 bytes that every pointer in the table is aligned to.
+hipError_t launch_copy_many(hipStream_t st, const CopyTable& t, int align, uint32_t max_blocks);
+
 // Plain device copy with the same packet shape (also the calibration kernel for
 // the memory counters): dst <- src, nbytes.
 hipError_t launch_copy(hipStream_t st, void* dst, const void* src, uint64_t nbytes,

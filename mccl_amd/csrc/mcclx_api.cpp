@@ -312,6 +312,48 @@ int ensure_slot(mcclx_ctx* ctx, TableSlot& sl, size_t need) {
     return MCCLX_OK;
 }
 
+// Puts a descriptor table where a kernel can read it (caller holds ctx->mu).
+// Outside a recording: the next slot of the pinned staging ring, copied to its
+// device twin on the queue; `*slot` must be handed to table_launched() after
+// the launch.  While recording: the launch needs a table that outlives this
+// call, so it gets its own device buffer, filled now with a blocking copy
+// (outside the recording) and owned by the graph; `*slot` stays null.
+int stage_table(mcclx_ctx* ctx, const void* bytes, size_t nbytes, void** dev, TableSlot** slot) {
+    *slot = nullptr;
+    if (ctx->capturing) {
+        void* d = nullptr;
+        HIP_TRY(hipMalloc(&d, nbytes));
+        // not the legacy stream: that one may not be touched while another stream records
+        if (!ctx->upload_stream)
+            HIP_TRY(hipStreamCreateWithFlags(&ctx->upload_stream, hipStreamNonBlocking));
+        hipError_t ce = hipMemcpyAsync(d, bytes, nbytes, hipMemcpyHostToDevice, ctx->upload_stream);
+        if (ce == hipSuccess) ce = hipStreamSynchronize(ctx->upload_stream);
+        if (ce != hipSuccess) {
+            (void)hipFree(d);
+            return fail(MCCLX_ERR_HIP, "table upload failed: %s", hipGetErrorString(ce));
+        }
+        ctx->capture_tables.push_back(d);
+        *dev = d;
+        return MCCLX_OK;
+    }
+    TableSlot& sl = ctx->slots[ctx->next_slot];
+    ctx->next_slot = (ctx->next_slot + 1) % kTableSlots;
+    if (int rc = ensure_slot(ctx, sl, nbytes)) return rc;
+    memcpy(sl.host, bytes, nbytes);
+    HIP_TRY(hipMemcpyAsync(sl.dev, sl.host, nbytes, hipMemcpyHostToDevice, ctx->stream));
+    *dev = sl.dev;
+    *slot = &sl;
+    return MCCLX_OK;
+}
+
+// The launch that reads the staged table has been issued: the slot is busy until it ends.
+int table_launched(mcclx_ctx* ctx, TableSlot* slot) {
+    if (!slot) return MCCLX_OK;
+    HIP_TRY(hipEventRecord(slot->done, ctx->stream));
+    slot->pending = true;
+    return MCCLX_OK;
+}
+
 int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uint32_t nseg) {
     if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
     mcclx::PlanKey key;
@@ -355,54 +397,9 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
     std::lock_guard<std::mutex> lk(ctx->mu);
     size_t seg_bytes = (size_t)nseg * sizeof(mcclx_seg);
     size_t pre_bytes = ((size_t)nseg + 1) * sizeof(uint64_t);
-    if (ctx->capturing) {
-        // A recorded launch needs a table that outlives this call: give it its
-        // own device buffer, filled now with a blocking copy (outside the
-        // recording), owned by the graph.
-        std::vector<char> host(seg_bytes + pre_bytes);
-        memcpy(host.data(), segs, seg_bytes);
-        uint64_t* pre = reinterpret_cast<uint64_t*>(host.data() + seg_bytes);
-        uint64_t total = 0, uniform = mcclx::items_for(key, segs[0].count);
-        for (uint32_t s = 0; s < nseg; ++s) {
-            pre[s] = total;
-            uint64_t n = mcclx::items_for(key, segs[s].count);
-            if (n != uniform) uniform = 0;
-            total += n;
-        }
-        pre[nseg] = total;
-        if (total == 0) return MCCLX_OK;
-        if (total >> 31) return fail(MCCLX_ERR_INVALID, "fold: more than 2^31 work items in one launch");
-        void* dev = nullptr;
-        HIP_TRY(hipMalloc(&dev, host.size()));
-        // not the legacy stream: that one may not be touched while another stream records
-        if (!ctx->upload_stream)
-            HIP_TRY(hipStreamCreateWithFlags(&ctx->upload_stream, hipStreamNonBlocking));
-        hipError_t ce = hipMemcpyAsync(dev, host.data(), host.size(), hipMemcpyHostToDevice,
-                                       ctx->upload_stream);
-        if (ce == hipSuccess) ce = hipStreamSynchronize(ctx->upload_stream);
-        if (ce != hipSuccess) {
-            (void)hipFree(dev);
-            return fail(MCCLX_ERR_HIP, "table upload failed: %s", hipGetErrorString(ce));
-        }
-        ctx->capture_tables.push_back(dev);
-        mcclx::TableArgs t;
-        t.segs = static_cast<const mcclx::SegArgs*>(dev);
-        t.first_item = reinterpret_cast<const uint64_t*>(static_cast<char*>(dev) + seg_bytes);
-        t.total_items = total;
-        t.uniform_items = uniform;
-        t.nseg = nseg;
-        t.scale = scale_f;
-        t.has_scale = has_scale;
-        lp.table = &t;
-        hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
-        if (e != hipSuccess) return launch_error(e, key);
-        return MCCLX_OK;
-    }
-    TableSlot& sl = ctx->slots[ctx->next_slot];
-    ctx->next_slot = (ctx->next_slot + 1) % kTableSlots;
-    if (int rc = ensure_slot(ctx, sl, seg_bytes + pre_bytes)) return rc;
-    memcpy(sl.host, segs, seg_bytes);
-    uint64_t* pre = reinterpret_cast<uint64_t*>(static_cast<char*>(sl.host) + seg_bytes);
+    std::vector<char> host(seg_bytes + pre_bytes);
+    memcpy(host.data(), segs, seg_bytes);
+    uint64_t* pre = reinterpret_cast<uint64_t*>(host.data() + seg_bytes);
     uint64_t total = 0, uniform = mcclx::items_for(key, segs[0].count);
     for (uint32_t s = 0; s < nseg; ++s) {
         pre[s] = total;
@@ -413,10 +410,12 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
     pre[nseg] = total;
     if (total == 0) return MCCLX_OK;
     if (total >> 31) return fail(MCCLX_ERR_INVALID, "fold: more than 2^31 work items in one launch");
-    HIP_TRY(hipMemcpyAsync(sl.dev, sl.host, seg_bytes + pre_bytes, hipMemcpyHostToDevice, ctx->stream));
+    void* dev = nullptr;
+    TableSlot* slot = nullptr;
+    if (int rc = stage_table(ctx, host.data(), host.size(), &dev, &slot)) return rc;
     mcclx::TableArgs t;
-    t.segs = static_cast<const mcclx::SegArgs*>(sl.dev);
-    t.first_item = reinterpret_cast<const uint64_t*>(static_cast<char*>(sl.dev) + seg_bytes);
+    t.segs = static_cast<const mcclx::SegArgs*>(dev);
+    t.first_item = reinterpret_cast<const uint64_t*>(static_cast<char*>(dev) + seg_bytes);
     t.total_items = total;
     t.uniform_items = uniform;
     t.nseg = nseg;
@@ -425,9 +424,7 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
     lp.table = &t;
     hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
     if (e != hipSuccess) return launch_error(e, key);
-    HIP_TRY(hipEventRecord(sl.done, ctx->stream));
-    sl.pending = true;
-    return MCCLX_OK;
+    return table_launched(ctx, slot);
 }
 
 int make_ctx(int device, hipStream_t borrowed, bool borrow, mcclx_ctx** out) {
@@ -606,6 +603,70 @@ int mcclx_copy(mcclx_ctx* ctx, void* dst, const void* src, uint64_t nbytes) {
     hipError_t e = mcclx::launch_copy(ctx->stream, dst, src, nbytes, ctx->max_blocks);
     if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "copy launch failed: %s", hipGetErrorString(e));
     return MCCLX_OK;
+}
+
+int mcclx_copy_batched(mcclx_ctx* ctx, const mcclx_copy_desc* descs, uint32_t n) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    if (n == 0) return MCCLX_OK;
+    if (!descs) return fail(MCCLX_ERR_INVALID, "copy_batched: descriptor array is null");
+    uintptr_t both = 0;
+    uint64_t bytes = 0;
+    uint32_t live = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        const mcclx_copy_desc& d = descs[i];
+        if (d.nbytes == 0 || d.dst == d.src) continue;
+        if (!d.dst || !d.src) return fail(MCCLX_ERR_INVALID, "copy_batched: descriptor %u has a null pointer", i);
+        if (ctx->validate) {
+            if (int rc = check_range(d.src, d.nbytes, "src", i)) return rc;
+            if (int rc = check_range(d.dst, d.nbytes, "dst", i)) return rc;
+        }
+        both |= reinterpret_cast<uintptr_t>(d.dst) | reinterpret_cast<uintptr_t>(d.src);
+        bytes += d.nbytes;
+        ++live;
+    }
+    if (live == 0) return MCCLX_OK;
+    DeviceGuard guard(ctx->device);
+    if (!guard.ok) return fail(MCCLX_ERR_HIP, "hipSetDevice(%d) failed", ctx->device);
+    // A few large copies: one launch each streams best (a block of the table kernel
+    // first has to fetch its descriptor from memory).  Many small ones: one launch.
+    if (live <= 4 || bytes / live >= (8u << 20)) {
+        for (uint32_t i = 0; i < n; ++i)
+            if (int rc = mcclx_copy(ctx, descs[i].dst, descs[i].src, descs[i].nbytes)) return rc;
+        return MCCLX_OK;
+    }
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    const size_t desc_bytes = (size_t)live * sizeof(mcclx::CopyDesc);
+    std::vector<char> host(desc_bytes + ((size_t)live + 1) * sizeof(uint64_t));
+    auto* hd = reinterpret_cast<mcclx::CopyDesc*>(host.data());
+    auto* pre = reinterpret_cast<uint64_t*>(host.data() + desc_bytes);
+    uint64_t total = 0, uniform = 0;
+    uint32_t j = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        const mcclx_copy_desc& d = descs[i];
+        if (d.nbytes == 0 || d.dst == d.src) continue;
+        hd[j] = mcclx::CopyDesc{d.dst, d.src, d.nbytes};
+        pre[j] = total;
+        const uint64_t items = mcclx::copy_items(d.nbytes);
+        if (j == 0) uniform = items;
+        if (items != uniform) uniform = 0;
+        total += items;
+        ++j;
+    }
+    pre[live] = total;
+    if (total >> 31) return fail(MCCLX_ERR_INVALID, "copy_batched: more than 2^31 work items in one launch");
+    void* dev = nullptr;
+    TableSlot* slot = nullptr;
+    if (int rc = stage_table(ctx, host.data(), host.size(), &dev, &slot)) return rc;
+    mcclx::CopyTable t;
+    t.descs = static_cast<const mcclx::CopyDesc*>(dev);
+    t.first_item = reinterpret_cast<const uint64_t*>(static_cast<char*>(dev) + desc_bytes);
+    t.total_items = (uint32_t)total;
+    t.uniform_items = (uint32_t)uniform;
+    t.n = live;
+    int align = (both % 4 == 0) ? 4 : (both % 2 == 0) ? 2 : 1;
+    hipError_t e = mcclx::launch_copy_many(ctx->stream, t, align, ctx->max_blocks);
+    if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "copy_batched launch failed: %s", hipGetErrorString(e));
+    return table_launched(ctx, slot);
 }
 
 int mcclx_batch_begin(mcclx_ctx* ctx, const char* label) {

@@ -197,66 +197,73 @@ mcclx_plan base_plan(const mcclx_replay* r, const Layout& L, int k) {
     return p;
 }
 
-int fold_any(mcclx_ctx* ctx, mcclx_plan p, std::vector<mcclx_seg>& segs) {
-    return mcclx_fold_batched(ctx, &p, segs.data(), (uint32_t)segs.size());
+// The launches of one or more fused allreduces that share a plan, gathered phase
+// by phase: what every rank encodes for the wire, the folds, the casts on
+// arrival, and the plain copies of the allgather leg.  Each phase is one launch.
+struct Phases {
+    bool planned = false;
+    mcclx_plan enc, fold, dec;
+    std::vector<mcclx_seg> enc_segs, fold_segs, dec_segs;
+    std::vector<mcclx_copy_desc> copies;
+};
+
+void plan_phases(const mcclx_replay* r, const Layout& L, Phases& ph) {
+    if (ph.planned) return;
+    ph.planned = true;
+    ph.fold = base_plan(r, L, r->world);
+    if (r->algo == MCCLX_ALGO_TREE) {
+        ph.fold.topo = MCCLX_TOPO_BINOMIAL;
+        if (L.wire) ph.fold.io = MCCLX_IO_OWN_FIRST_F32;
+    } else if (L.wire) {
+        ph.fold.io = r->algo == MCCLX_ALGO_RING ? MCCLX_IO_OWN_LAST_F32 : MCCLX_IO_OWN_FIRST_F32;
+    }
+    ph.enc = base_plan(r, L, 1);  // fp32 -> bf16 of what travels
+    ph.enc.io = MCCLX_IO_OWN_FIRST_F32;
+    ph.enc.op = MCCLX_SUM;
+    ph.enc.scale_mode = MCCLX_SCALE_NONE;
+    ph.dec = ph.enc;              // bf16 -> fp32 on arrival
+    ph.dec.io = MCCLX_IO_OUT_F32;
 }
 
-int replay_fused(mcclx_ctx* ctx, const mcclx_replay* r, const Layout& L) {
+void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
+    plan_phases(r, L, ph);
     const int N = r->world;
     const uint64_t es = esize(L.wdtype);  // element size on the "wire"
     const uint64_t ts = esize(r->dtype);  // element size of the rank tensors
     auto wire_of = [&](int rank) -> void* { return at(r->workspace, (uint64_t)rank * L.wire_stride); };
-    std::vector<mcclx_seg> segs;
     mcclx_seg z;
     memset(&z, 0, sizeof z);
 
     if (r->algo == MCCLX_ALGO_TREE) {
         // allreduce_tree: rank 0 ends with the binomial combination of all
         // tensors (AllreduceAlgos.cpp:100-114), everyone else receives a copy.
-        mcclx_plan p = base_plan(r, L, N);
-        p.topo = MCCLX_TOPO_BINOMIAL;
-        if (L.wire) {
-            mcclx_plan e = base_plan(r, L, 1);  // encode ranks 1.. (their tensors travel)
-            e.io = MCCLX_IO_OWN_FIRST_F32;
-            e.op = MCCLX_SUM;
-            e.scale_mode = MCCLX_SCALE_NONE;
-            for (int q = 1; q < N; ++q) {
+        if (L.wire)
+            for (int q = 1; q < N; ++q) {  // ranks 1.. encode: their tensors travel
                 mcclx_seg s = z;
                 s.wire_out = wire_of(q);
                 s.in[0] = r->tensors[q];
                 s.count = r->numel;
-                segs.push_back(s);
+                ph.enc_segs.push_back(s);
             }
-            if (!segs.empty()) TRY(mcclx_fold_batched(ctx, &e, segs.data(), (uint32_t)segs.size()));
-            segs.clear();
-            p.io = MCCLX_IO_OWN_FIRST_F32;
-        }
         mcclx_seg s = z;
         s.out = r->tensors[0];
         s.count = r->numel;
         s.in[0] = r->tensors[0];
         for (int q = 1; q < N; ++q) s.in[q] = L.wire ? wire_of(q) : r->tensors[q];
         if (L.wire) s.wire_out = wire_of(0);
-        segs.push_back(s);
-        TRY(fold_any(ctx, p, segs));
-        segs.clear();
-        if (L.wire) {  // broadcast of the bf16 result + the final cast on every rank
-            mcclx_plan d = base_plan(r, L, 1);
-            d.io = MCCLX_IO_OUT_F32;
-            d.op = MCCLX_SUM;
-            d.scale_mode = MCCLX_SCALE_NONE;
-            for (int q = 1; q < N; ++q) {
+        ph.fold_segs.push_back(s);
+        for (int q = 1; q < N; ++q) {
+            if (L.wire) {  // broadcast of the bf16 result + the final cast on every rank
                 mcclx_seg g = z;
                 g.out = r->tensors[q];
                 g.in[0] = wire_of(0);
                 g.count = r->numel;
-                segs.push_back(g);
+                ph.dec_segs.push_back(g);
+            } else {
+                ph.copies.push_back(mcclx_copy_desc{r->tensors[q], r->tensors[0], r->numel * ts});
             }
-            if (!segs.empty()) TRY(mcclx_fold_batched(ctx, &d, segs.data(), (uint32_t)segs.size()));
-        } else {
-            for (int q = 1; q < N; ++q) TRY(mcclx_copy(ctx, r->tensors[q], r->tensors[0], r->numel * ts));
         }
-        return MCCLX_OK;
+        return;
     }
 
     // ring and butterfly: chunk c has one final owner who folds all N operands.
@@ -271,12 +278,7 @@ int replay_fused(mcclx_ctx* ctx, const mcclx_replay* r, const Layout& L) {
         return (j - 1 < chunk) ? j - 1 : j;  // ascending peers, skipping the owner
     };
 
-    if (L.wire) {
-        // every rank encodes what it sends: all chunks except the one it owns
-        mcclx_plan e = base_plan(r, L, 1);
-        e.io = MCCLX_IO_OWN_FIRST_F32;
-        e.op = MCCLX_SUM;
-        e.scale_mode = MCCLX_SCALE_NONE;
+    if (L.wire)  // every rank encodes what it sends: all chunks except the one it owns
         for (int q = 0; q < N; ++q)
             for (int ch = 0; ch < N; ++ch) {
                 if (owner_of(ch) == q || c[ch].elem_count == 0) continue;
@@ -284,14 +286,9 @@ int replay_fused(mcclx_ctx* ctx, const mcclx_replay* r, const Layout& L) {
                 s.wire_out = at(wire_of(q), (uint64_t)c[ch].elem_start * 2);
                 s.in[0] = at(r->tensors[q], (uint64_t)c[ch].elem_start * 4);
                 s.count = (uint64_t)c[ch].elem_count;
-                segs.push_back(s);
+                ph.enc_segs.push_back(s);
             }
-        if (!segs.empty()) TRY(mcclx_fold_batched(ctx, &e, segs.data(), (uint32_t)segs.size()));
-        segs.clear();
-    }
 
-    mcclx_plan p = base_plan(r, L, N);
-    if (L.wire) p.io = ring ? MCCLX_IO_OWN_LAST_F32 : MCCLX_IO_OWN_FIRST_F32;
     for (int ch = 0; ch < N; ++ch) {
         if (c[ch].elem_count == 0) continue;
         int o = owner_of(ch);
@@ -306,43 +303,86 @@ int replay_fused(mcclx_ctx* ctx, const mcclx_replay* r, const Layout& L) {
             else
                 s.in[j] = at(r->tensors[q], (uint64_t)c[ch].elem_start * ts);
         }
-        segs.push_back(s);
+        ph.fold_segs.push_back(s);
     }
-    TRY(fold_any(ctx, p, segs));
-    segs.clear();
 
     // allgather leg (AllreduceAlgos.cpp:77-86,185-200): every other rank gets
     // the owner's reduced chunk; with the wire codec it arrives as bf16 and is
     // cast on arrival (ProcessGroupMCCL.cpp:179-183).
-    if (L.wire) {
-        mcclx_plan d = base_plan(r, L, 1);
-        d.io = MCCLX_IO_OUT_F32;
-        d.op = MCCLX_SUM;
-        d.scale_mode = MCCLX_SCALE_NONE;
-        for (int ch = 0; ch < N; ++ch) {
-            if (c[ch].elem_count == 0) continue;
-            int o = owner_of(ch);
-            for (int q = 0; q < N; ++q) {
-                if (q == o) continue;
+    for (int ch = 0; ch < N; ++ch) {
+        if (c[ch].elem_count == 0) continue;
+        int o = owner_of(ch);
+        for (int q = 0; q < N; ++q) {
+            if (q == o) continue;
+            if (L.wire) {
                 mcclx_seg s = z;
                 s.out = at(r->tensors[q], (uint64_t)c[ch].elem_start * 4);
                 s.in[0] = at(wire_of(o), (uint64_t)c[ch].elem_start * 2);
                 s.count = (uint64_t)c[ch].elem_count;
-                segs.push_back(s);
+                ph.dec_segs.push_back(s);
+            } else {
+                ph.copies.push_back(mcclx_copy_desc{at(r->tensors[q], (uint64_t)c[ch].elem_start * ts),
+                                                    at(r->tensors[o], (uint64_t)c[ch].elem_start * ts),
+                                                    (uint64_t)c[ch].elem_count * ts});
             }
         }
-        if (!segs.empty()) TRY(mcclx_fold_batched(ctx, &d, segs.data(), (uint32_t)segs.size()));
-    } else {
-        for (int ch = 0; ch < N; ++ch) {
-            int o = owner_of(ch);
-            for (int q = 0; q < N; ++q)
-                if (q != o)
-                    TRY(mcclx_copy(ctx, at(r->tensors[q], (uint64_t)c[ch].elem_start * ts),
-                                   at(r->tensors[o], (uint64_t)c[ch].elem_start * ts),
-                                   (uint64_t)c[ch].elem_count * ts));
-        }
     }
+}
+
+int issue_phases(mcclx_ctx* ctx, Phases& ph) {
+    if (!ph.enc_segs.empty())
+        TRY(mcclx_fold_batched(ctx, &ph.enc, ph.enc_segs.data(), (uint32_t)ph.enc_segs.size()));
+    if (!ph.fold_segs.empty())
+        TRY(mcclx_fold_batched(ctx, &ph.fold, ph.fold_segs.data(), (uint32_t)ph.fold_segs.size()));
+    if (!ph.dec_segs.empty())
+        TRY(mcclx_fold_batched(ctx, &ph.dec, ph.dec_segs.data(), (uint32_t)ph.dec_segs.size()));
+    if (!ph.copies.empty()) TRY(mcclx_copy_batched(ctx, ph.copies.data(), (uint32_t)ph.copies.size()));
     return MCCLX_OK;
+}
+
+// Argument checks of one replay; *fused says whether the fused schedule can run it.
+int check_replay(mcclx_ctx* ctx, const mcclx_replay* r, bool* fused, bool* nothing_to_do) {
+    *fused = false;
+    *nothing_to_do = false;
+    if (!ctx || !r || !r->tensors) return bad("replay: null argument");
+    if (r->world < 1 || r->reserved != 0) return bad("replay: bad world");
+    if (r->algo < MCCLX_ALGO_RING || r->algo > MCCLX_ALGO_BUTTERFLY) return bad("replay: bad algo");
+    if (r->mode != MCCLX_REPLAY_STEPWISE && r->mode != MCCLX_REPLAY_FUSED) return bad("replay: bad mode");
+    if (r->op < MCCLX_SUM || r->op > MCCLX_MAX) {
+        // surfaces "Unsupported ReduceOp: n" through the kernel layer
+        return mcclx_reduce(ctx, r->tensors[0], r->tensors[0], r->dtype, 0, r->op);
+    }
+    if (r->world == 1) {  // ProcessGroupMCCL.cpp:107
+        *nothing_to_do = true;
+        return MCCLX_OK;
+    }
+    if (r->numel == 0) return bad("replay: empty tensor");  // TensorChecks.hpp:31-34
+    // AllreduceAlgos.cpp:55,137
+    if (r->algo != MCCLX_ALGO_TREE && r->numel < (uint64_t)r->world) return bad("numel must be >= world");
+    for (int i = 0; i < r->world; ++i)
+        if (!r->tensors[i]) return bad("replay: null tensor");
+    Layout L = layout_of(r);
+    if (L.total > 0 && (!r->workspace || r->workspace_bytes < L.total)) return bad("workspace too small");
+    bool f = r->mode == MCCLX_REPLAY_FUSED && r->world <= MCCLX_MAX_INPUTS;
+    // The wire codec mixes fp32 and bf16 operands, which only the SUM fold
+    // handles; MIN / MAX / PRODUCT over the wire run the stepwise schedule.
+    if (f && L.wire && r->op != MCCLX_SUM && r->op != MCCLX_AVG) f = false;
+    *fused = f;
+    return MCCLX_OK;
+}
+
+int run_stepwise(mcclx_ctx* ctx, const mcclx_replay* r) {
+    mcclx_replay s = *r;
+    s.mode = MCCLX_REPLAY_STEPWISE;
+    Layout Ls = layout_of(&s);
+    if (Ls.total > 0 && (!r->workspace || r->workspace_bytes < Ls.total)) return bad("workspace too small");
+    return replay_stepwise(ctx, &s, Ls);
+}
+
+// Same plan for every phase?
+bool same_plan(const mcclx_replay* a, const mcclx_replay* b) {
+    return a->world == b->world && a->algo == b->algo && a->op == b->op && a->dtype == b->dtype &&
+           (a->wire_bf16 != 0) == (b->wire_bf16 != 0) && a->acc == b->acc;
 }
 
 }  // namespace
@@ -384,35 +424,39 @@ uint64_t mcclx_replay_workspace_bytes(const mcclx_replay* r) {
 }
 
 int mcclx_allreduce_replay(mcclx_ctx* ctx, const mcclx_replay* r) {
-    if (!ctx || !r || !r->tensors) return bad("replay: null argument");
-    if (r->world < 1 || r->reserved != 0) return bad("replay: bad world");
-    if (r->algo < MCCLX_ALGO_RING || r->algo > MCCLX_ALGO_BUTTERFLY) return bad("replay: bad algo");
-    if (r->mode != MCCLX_REPLAY_STEPWISE && r->mode != MCCLX_REPLAY_FUSED) return bad("replay: bad mode");
-    if (r->op < MCCLX_SUM || r->op > MCCLX_MAX) {
-        // surfaces "Unsupported ReduceOp: n" through the kernel layer
-        return mcclx_reduce(ctx, r->tensors[0], r->tensors[0], r->dtype, 0, r->op);
-    }
-    if (r->world == 1) return MCCLX_OK;  // ProcessGroupMCCL.cpp:107
-    if (r->numel == 0) return bad("replay: empty tensor");  // TensorChecks.hpp:31-34
-    // AllreduceAlgos.cpp:55,137
-    if (r->algo != MCCLX_ALGO_TREE && r->numel < (uint64_t)r->world) return bad("numel must be >= world");
-    for (int i = 0; i < r->world; ++i)
-        if (!r->tensors[i]) return bad("replay: null tensor");
-    Layout L = layout_of(r);
-    if (L.total > 0 && (!r->workspace || r->workspace_bytes < L.total)) return bad("workspace too small");
+    return mcclx_allreduce_replay_many(ctx, r, 1);
+}
 
-    bool fused = r->mode == MCCLX_REPLAY_FUSED && r->world <= MCCLX_MAX_INPUTS;
-    // The wire codec mixes fp32 and bf16 operands, which only the SUM fold
-    // handles; MIN / MAX / PRODUCT over the wire run the stepwise schedule.
-    if (fused && L.wire && r->op != MCCLX_SUM && r->op != MCCLX_AVG) fused = false;
-    if (!fused) {
-        mcclx_replay s = *r;
-        s.mode = MCCLX_REPLAY_STEPWISE;
-        Layout Ls = layout_of(&s);
-        if (Ls.total > 0 && (!r->workspace || r->workspace_bytes < Ls.total)) return bad("workspace too small");
-        return replay_stepwise(ctx, &s, Ls);
+int mcclx_allreduce_replay_many(mcclx_ctx* ctx, const mcclx_replay* rs, uint32_t n) {
+    if (n && !rs) return bad("replay: null argument");
+    uint32_t i = 0;
+    while (i < n) {
+        bool fused, nothing;
+        TRY(check_replay(ctx, &rs[i], &fused, &nothing));
+        if (nothing) {
+            ++i;
+            continue;
+        }
+        if (!fused) {
+            TRY(run_stepwise(ctx, &rs[i]));
+            ++i;
+            continue;
+        }
+        // gather the run of fused replays that share this one's plan
+        Phases ph;
+        const mcclx_replay* first = &rs[i];
+        while (i < n) {
+            if (&rs[i] != first) {
+                if (!same_plan(first, &rs[i])) break;
+                TRY(check_replay(ctx, &rs[i], &fused, &nothing));
+                if (!fused || nothing) break;
+            }
+            collect_fused(&rs[i], layout_of(&rs[i]), ph);
+            ++i;
+        }
+        TRY(issue_phases(ctx, ph));
     }
-    return replay_fused(ctx, r, L);
+    return MCCLX_OK;
 }
 
 int mcclx_reduce_scatter_shares(mcclx_ctx* ctx, int world, void* const* outs,
@@ -455,7 +499,7 @@ int mcclx_reduce_scatter_shares(mcclx_ctx* ctx, int world, void* const* outs,
         for (int q = 0; q < world; ++q)
             if (q != r) segs[r].in[j++] = share(r, q);  // ascending peers (:379-383)
     }
-    return fold_any(ctx, p, segs);
+    return mcclx_fold_batched(ctx, &p, segs.data(), (uint32_t)segs.size());
 }
 
 int mcclx_reduce_scatter_replay(mcclx_ctx* ctx, int world, void* const* outs,

@@ -121,6 +121,43 @@ def allreduce_replay(tensors: List[torch.Tensor], op, algo: int, wire_bf16: bool
         own_ws.free()
 
 
+def allreduce_replay_many(groups: List[List[torch.Tensor]], op, algo: int, wire_bf16: bool = False,
+                          mode: int = L.REPLAY_FUSED, acc: int = L.ACC_STEP, queue=None) -> None:
+    """A list of allreduces (groups[i] = the virtual ranks' tensors of message i), as a
+    c10d allreduce over a list of tensors: entries that share a plan go out together,
+    one launch per phase for all of them."""
+    q = _q(queue)
+    reps = (L.Replay * len(groups))()
+    keep = []
+    needs = []
+    for i, tensors in enumerate(groups):
+        for t in tensors:
+            _check_tensor(t, "allreduce")
+        r = reps[i]
+        r.world = len(tensors)
+        r.algo, r.op, r.dtype = algo, op_code(op), dtype_code(tensors[0])
+        r.wire_bf16, r.mode, r.acc, r.reserved = int(wire_bf16), L.REPLAY_STEPWISE, acc, 0
+        r.numel = tensors[0].numel()
+        ptrs = _ptr_array([t.data_ptr() for t in tensors])
+        keep.append(ptrs)
+        r.tensors = ptrs
+        need = L.lib().mcclx_replay_workspace_bytes(C.byref(r))     # stepwise needs the most
+        r.mode = mode
+        needs.append((max(need, L.lib().mcclx_replay_workspace_bytes(C.byref(r))) + 255) // 256 * 256)
+    ws = Workspace(q, sum(needs))
+    off = 0
+    for i, need in enumerate(needs):
+        reps[i].workspace = (ws.ptr + off) or None
+        reps[i].workspace_bytes = need
+        off += need
+    q.wait_torch_stream()
+    try:
+        L.check(L.lib().mcclx_allreduce_replay_many(q.handle, reps, len(groups)))
+    finally:
+        q.drain()
+        ws.free()
+
+
 def allreduce(tensors: List[torch.Tensor], op="sum", queue=None, mode: int = L.REPLAY_FUSED) -> int:
     """ProcessGroupMCCL::allreduce for N virtual ranks; returns the algorithm used."""
     wire, env_algo, tree_below = _env_config()

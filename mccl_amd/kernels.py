@@ -181,6 +181,11 @@ class ReduceQueue:
     def copy(self, dst_ptr: int, src_ptr: int, nbytes: int) -> None:
         L.check(L.lib().mcclx_copy(self.handle, C.c_void_p(dst_ptr), C.c_void_p(src_ptr), nbytes))
 
+    def copy_batched(self, triples) -> None:
+        """Many (dst, src, nbytes) copies in one launch (a few large ones go out one by one)."""
+        arr = (L.CopyDesc * len(triples))(*[L.CopyDesc(d, s, n) for d, s, n in triples])
+        L.check(L.lib().mcclx_copy_batched(self.handle, arr, len(triples)))
+
 
 _default: Optional[ReduceQueue] = None
 _batch_depth_owner = None

@@ -561,3 +561,30 @@ def test_graph_cache_can_be_switched_off(CX, monkeypatch):
     out, errs = run_ranks(CX, 2, fn)
     assert errs == [None, None], errs
     assert out == [0, 0]
+
+
+def test_allreduce_of_a_long_tensor_list_goes_out_together(CX, U, monkeypatch):
+    """The C4 shape through the c10d surface: one allreduce call over a list of 600 small
+    messages (tree, since each is below MCCL_TREE_BELOW) plus a few larger ones (ring);
+    every message bit-exact against the oracle's replay of the reference."""
+    world = 3
+    monkeypatch.delenv("MCCL_ALLREDUCE_ALGO", raising=False)
+    monkeypatch.delenv("MCCL_WIRE_DTYPE", raising=False)
+    monkeypatch.delenv("MCCL_TREE_BELOW", raising=False)
+    rng = np.random.default_rng(404)
+    sizes = [16384] * 200 + [int(n) for n in rng.integers(1, 5000, 400)] + [70000, 100003]
+    host = [[U.rand_values(rng, n, F32, scale=1.0) for _ in range(world)] for n in sizes]
+
+    def fn(r, pg):
+        ts = [U.to_dev(msg[r], F32) for msg in host]
+        pg.allreduce(ts).wait()
+        return [U.bits(t) for t in ts]
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for i, (n, msg) in enumerate(zip(sizes, host)):
+        want = [x.copy() for x in msg]
+        rc, used = orc.pg_allreduce(want, F32, SUM)
+        assert rc == 0 and used == (TREE if n * 4 <= 262144 else RING)
+        for r in range(world):
+            assert np.array_equal(out[r][i], want[r].view(np.uint32)), (i, n, r)

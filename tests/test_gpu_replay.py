@@ -205,3 +205,46 @@ def test_f32acc_reduce_scatter_variant(H, U):
     H.reduce_scatter_replay(dout, din, SUM, mode=FUSED, acc=1)
     for r in range(world):
         assert np.array_equal(U.bits(dout[r]), want[r])
+
+
+@pytest.mark.parametrize("algo", [RING, TREE, BUTTERFLY])
+@pytest.mark.parametrize("dtype,wire", [(F32, False), (BF16, False), (F32, True)])
+def test_many_messages_in_one_replay_equal_single_replays(H, U, algo, dtype, wire):
+    """A list of allreduces issued together (one launch per phase for all of them) gives
+    what the oracle gives for each message on its own: mixed sizes, more messages than fit
+    the kernel arguments, world 3."""
+    world = 3
+    rng = np.random.default_rng(17 + algo)
+    sizes = [3, 5, 64, 997, 4099, 16384, 16384, 33, 70001] + [int(n) for n in rng.integers(3, 3000, 40)]
+    host = [[U.rand_values(rng, n, dtype, scale=1e-2, specials=(n > 64)) for _ in range(world)] for n in sizes]
+    groups = [[U.to_dev(x, dtype) for x in msg] for msg in host]
+    H.allreduce_replay_many(groups, "avg" if dtype == F32 else "sum", algo, wire_bf16=wire)
+    for n, msg, g in zip(sizes, host, groups):
+        want = [x.copy() for x in msg]
+        op = AVG if dtype == F32 else SUM
+        rc = orc.allreduce(algo, want, dtype, op) if not wire else \
+            orc.pg_allreduce(want, dtype, op, wire_bf16=True, env_algo={RING: "ring", TREE: "tree", BUTTERFLY: "butterfly"}[algo])[0]
+        assert rc == 0
+        for r in range(world):
+            U.assert_same_bits(g[r], want[r], dtype, f"algo {algo} n {n} rank {r}")
+
+
+def test_copy_batched_many_small_and_a_few_large(K, U):
+    rng = np.random.default_rng(3)
+    q = K._q(None)
+    for sizes in ([int(n) for n in rng.integers(1, 70000, 300)], [1, 2, 3, 15, 16, 17], [20_000_001, 9_000_003, 5, 0, 7]):
+        total = sum(sizes) + 64 * len(sizes)
+        src = torch.randint(0, 256, (total,), dtype=torch.uint8, device="cuda")
+        dst = torch.zeros(total, dtype=torch.uint8, device="cuda")
+        want = np.zeros(total, np.uint8)
+        hs = src.cpu().numpy()
+        triples, off = [], 0
+        for i, n in enumerate(sizes):
+            so, do = off + int(rng.integers(0, 16)), off + int(rng.integers(0, 16))
+            triples.append((dst.data_ptr() + do, src.data_ptr() + so, n))
+            want[do:do + n] = hs[so:so + n]
+            off += n + 64
+        torch.cuda.synchronize()
+        q.copy_batched(triples)
+        q.drain()
+        assert np.array_equal(dst.cpu().numpy(), want), sizes[:5]
