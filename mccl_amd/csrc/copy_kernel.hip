@@ -80,6 +80,10 @@ __global__ void __launch_bounds__(kBlock) copy_many_kernel(CopyTable t) {
         if (t.uniform_items) {  // every copy has the same number of tiles: no search
             c = w / t.uniform_items;
             tile = w - c * t.uniform_items;
+        } else if (t.item_map) {
+            const uint2 m = t.item_map[w];
+            c = m.x;
+            tile = m.y;
         } else {
             uint32_t lo = 0, hi = t.n;  // first_item[lo] <= w < first_item[hi]
             while (hi - lo > 1) {

@@ -481,6 +481,10 @@ __global__ void __launch_bounds__(kBlock) fold_table_kernel(TableArgs a) {
         if (uniform) {
             seg = w / uniform;
             tile = w - seg * uniform;
+        } else if (a.item_map) {  // ragged segments: the host has written out who owns item w
+            const uint2 m = a.item_map[w];
+            seg = m.x;
+            tile = m.y;
         } else {
             uint32_t lo = 0, hi = a.nseg;  // first_item[lo] <= w < first_item[hi]
             while (hi - lo > 1) {

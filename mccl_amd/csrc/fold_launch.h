@@ -36,6 +36,7 @@ struct FewArgs {
 struct TableArgs {
     const SegArgs* __restrict__ segs;         // device memory, nseg entries
     const uint64_t* __restrict__ first_item;  // device memory, nseg+1 prefix sums (unused when uniform)
+    const uint2* __restrict__ item_map;       // device memory, (segment, tile) of every work item, or null
     uint64_t total_items;
     uint64_t uniform_items;      // >0: every segment has this many work items
     uint32_t nseg;
@@ -70,6 +71,7 @@ struct CopyDesc {
 struct CopyTable {
     const CopyDesc* __restrict__ descs;
     const uint64_t* __restrict__ first_item;
+    const uint2* __restrict__ item_map;  // (copy, tile) of every work item, or null
     uint32_t total_items;
     uint32_t uniform_items;  // >0: every copy has this many work items
     uint32_t n;
