@@ -1,16 +1,13 @@
-// ProcessGroupMCCL.hpp -- the c10d Backend surface of the reference
-// (csrc/backend/ProcessGroupMCCL.hpp:43-94) for ROCm tensors.
+// ProcessGroupMCCL.hpp -- backend "mccl" for ROCm tensors: the c10d::Backend
+// surface of the reference (csrc/backend/ProcessGroupMCCL.hpp:43-94) over the
+// reduce + wire-codec path in libmcclx.
 //
-// Same virtuals, same option structs, same error behaviour; the work behind
-// them is the reduce + wire-codec path in libmcclx (C ABI), reached through
-// the chunk scheduler.  A group of size 1 completes every collective at once,
-// like the reference.  A group of size N > 1 lives inside one process on one
-// GPU: its ranks meet in a LocalMesh instead of over TCP.
-//
-// In scope: allreduce, reduce_scatter (+ _base), allgather (+ _base), plus
-// broadcast and barrier (pure copies / a rendezvous, needed by callers such as
-// DistributedDataParallel).  alltoall, send and recv move bytes between
-// processes without any arithmetic; they return a failed Work here.
+// The collectives keep the reference's observable behaviour (which run on the
+// caller's thread, which on the FIFO engine, what fails how).  What differs is
+// underneath: a group of N > 1 ranks lives inside one process on one GPU, its
+// ranks meet in a LocalMesh instead of over TCP, and the last rank to arrive
+// launches the device work of the whole group through the chunk scheduler.
+// A group of size 1 completes every collective at once, like the reference.
 #pragma once
 
 #include <torch/csrc/distributed/c10d/Backend.hpp>
@@ -21,6 +18,7 @@
 #include <ATen/ATen.h>
 
 #include <chrono>
+#include <functional>
 #include <memory>
 #include <string>
 #include <vector>
@@ -34,6 +32,10 @@ class LocalMesh;
 struct Contribution;
 
 class ProcessGroupMCCL : public c10d::Backend {
+    using Tensors = std::vector<at::Tensor>;
+    using TensorLists = std::vector<std::vector<at::Tensor>>;
+    using WorkPtr = c10::intrusive_ptr<c10d::Work>;
+
 public:
     struct Options {
         std::chrono::milliseconds timeout{30 * 60 * 1000};
@@ -44,30 +46,24 @@ public:
 
     const std::string getBackendName() const override { return "mccl"; }
 
-    c10::intrusive_ptr<c10d::Work> allreduce(std::vector<at::Tensor>& tensors,
-                                             const c10d::AllreduceOptions& opts = {}) override;
-    c10::intrusive_ptr<c10d::Work> broadcast(std::vector<at::Tensor>& tensors,
-                                             const c10d::BroadcastOptions& opts = {}) override;
-    c10::intrusive_ptr<c10d::Work> allgather(std::vector<std::vector<at::Tensor>>& output_tensors,
-                                             std::vector<at::Tensor>& input_tensors,
-                                             const c10d::AllgatherOptions& opts = {}) override;
-    c10::intrusive_ptr<c10d::Work> _allgather_base(at::Tensor& output_tensor, at::Tensor& input_tensor,
-                                                   const c10d::AllgatherOptions& opts = {}) override;
-    c10::intrusive_ptr<c10d::Work> reduce_scatter(std::vector<at::Tensor>& output_tensors,
-                                                  std::vector<std::vector<at::Tensor>>& input_tensors,
-                                                  const c10d::ReduceScatterOptions& opts = {}) override;
-    c10::intrusive_ptr<c10d::Work> _reduce_scatter_base(at::Tensor& output_tensor, at::Tensor& input_tensor,
-                                                        const c10d::ReduceScatterOptions& opts = {}) override;
-    c10::intrusive_ptr<c10d::Work> alltoall_base(at::Tensor& output_tensor, at::Tensor& input_tensor,
-                                                 std::vector<int64_t>& output_split_sizes,
-                                                 std::vector<int64_t>& input_split_sizes,
-                                                 const c10d::AllToAllOptions& opts = {}) override;
-    c10::intrusive_ptr<c10d::Work> alltoall(std::vector<at::Tensor>& output_tensors,
-                                            std::vector<at::Tensor>& input_tensors,
-                                            const c10d::AllToAllOptions& opts = {}) override;
-    c10::intrusive_ptr<c10d::Work> barrier(const c10d::BarrierOptions& opts = {}) override;
-    c10::intrusive_ptr<c10d::Work> send(std::vector<at::Tensor>& tensors, int dst_rank, int tag) override;
-    c10::intrusive_ptr<c10d::Work> recv(std::vector<at::Tensor>& tensors, int src_rank, int tag) override;
+    // reductions: the hot path.  allreduce blocks and returns a finished Work
+    // (ProcessGroupMCCL.cpp:105-186); the others run on the engine thread.
+    WorkPtr allreduce(Tensors& tensors, const c10d::AllreduceOptions& opts = {}) override;
+    WorkPtr _reduce_scatter_base(at::Tensor& output, at::Tensor& input,
+                                 const c10d::ReduceScatterOptions& opts = {}) override;
+    WorkPtr reduce_scatter(Tensors& outputs, TensorLists& inputs,
+                           const c10d::ReduceScatterOptions& opts = {}) override;
+
+    // data movement between the ranks of the group
+    WorkPtr _allgather_base(at::Tensor& output, at::Tensor& input, const c10d::AllgatherOptions& opts = {}) override;
+    WorkPtr allgather(TensorLists& outputs, Tensors& inputs, const c10d::AllgatherOptions& opts = {}) override;
+    WorkPtr broadcast(Tensors& tensors, const c10d::BroadcastOptions& opts = {}) override;
+    WorkPtr alltoall_base(at::Tensor& output, at::Tensor& input, std::vector<int64_t>& output_split_sizes,
+                          std::vector<int64_t>& input_split_sizes, const c10d::AllToAllOptions& opts = {}) override;
+    WorkPtr alltoall(Tensors& outputs, Tensors& inputs, const c10d::AllToAllOptions& opts = {}) override;
+    WorkPtr send(Tensors& tensors, int dst_rank, int tag) override;
+    WorkPtr recv(Tensors& tensors, int src_rank, int tag) override;
+    WorkPtr barrier(const c10d::BarrierOptions& opts = {}) override;
 
     // Algorithm the last allreduce on this rank ran (MCCLX_ALGO_*), for tests.
     int lastAlgo() const { return last_algo_; }
@@ -75,7 +71,7 @@ public:
     uint64_t graphHits() const;
 
 private:
-    struct Shared;  // reduce queue + scratch shared by the ranks of one mesh
+    struct Shared;  // reduce queue, scratch and recorded graphs shared by the ranks of one mesh
 
     void meet(Contribution c, const std::function<void(const std::vector<Contribution>&)>& leader);
     void meet_built(int kind, void* stream, const std::function<void(Contribution&)>& build,

@@ -2,24 +2,80 @@
 
 #include <ATen/core/ivalue.h>
 
+#include "backend/Errors.hpp"
+
 namespace mccl {
 
-WorkMCCL::WorkMCCL(c10d::OpType op, std::vector<at::Tensor> outputs, const char* title)
-    : c10d::Work(/*rank=*/-1, op, title, outputs), outputs_(std::move(outputs)) {
+namespace {
+
+// The Future must know which devices its value lives on.
+std::vector<c10::Device> devices_of(const std::vector<at::Tensor>& tensors) {
     std::vector<c10::Device> devices;
-    for (const auto& t : outputs_)
+    for (const at::Tensor& t : tensors)
         if (t.defined() && t.device().has_index()) devices.push_back(t.device());
-    future_ = c10::make_intrusive<c10::ivalue::Future>(c10::ListType::create(c10::TensorType::get()),
-                                                       devices);
+    return devices;
 }
+
+}  // namespace
+
+WorkMCCL::WorkMCCL(c10d::OpType op, std::vector<at::Tensor> outputs, const char* title)
+    : c10d::Work(/*rank=*/-1, op, title, outputs),
+      outputs_(std::move(outputs)),
+      future_(c10::make_intrusive<c10::ivalue::Future>(c10::ListType::create(c10::TensorType::get()),
+                                                       devices_of(outputs_))) {}
 
 WorkMCCL::~WorkMCCL() = default;
 
-bool WorkMCCL::isCompleted() { return done_.load(std::memory_order_acquire); }
+void WorkMCCL::settle(std::exception_ptr error) {
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        if (state_ != State::Pending) return;
+        error_ = error;
+        state_ = error ? State::Failed : State::Succeeded;
+    }
+    // outside the lock: the Future runs its callbacks inline
+    if (error)
+        future_->setError(error);
+    else
+        future_->markCompleted(c10::IValue(outputs_));
+    settled_cv_.notify_all();
+}
+
+void WorkMCCL::finish() {
+    std::exception_ptr failure;
+    if (before_done_) {
+        try {
+            before_done_();
+        } catch (...) {
+            failure = std::current_exception();  // a failed drain fails the collective
+        }
+    }
+    settle(failure);
+}
+
+void WorkMCCL::finishWithException(std::exception_ptr error) {
+    settle(error ? error : std::make_exception_ptr(MCCLError("collective failed without an error object")));
+}
+
+bool WorkMCCL::wait(std::chrono::milliseconds timeout) {
+    std::unique_lock<std::mutex> lk(mu_);
+    const auto settled = [this] { return state_ != State::Pending; };
+    if (timeout == kNoTimeout)
+        settled_cv_.wait(lk, settled);
+    else if (!settled_cv_.wait_for(lk, timeout, settled))
+        return false;
+    if (state_ == State::Failed) std::rethrow_exception(error_);
+    return true;
+}
+
+bool WorkMCCL::isCompleted() {
+    std::lock_guard<std::mutex> lk(mu_);
+    return state_ != State::Pending;
+}
 
 bool WorkMCCL::isSuccess() const {
     std::lock_guard<std::mutex> lk(mu_);
-    return done_.load(std::memory_order_acquire) && !error_;
+    return state_ == State::Succeeded;
 }
 
 std::exception_ptr WorkMCCL::exception() const {
@@ -27,48 +83,8 @@ std::exception_ptr WorkMCCL::exception() const {
     return error_;
 }
 
-bool WorkMCCL::wait(std::chrono::milliseconds timeout) {
-    std::unique_lock<std::mutex> lk(mu_);
-    auto finished = [this] { return done_.load(std::memory_order_acquire); };
-    if (timeout == kNoTimeout)
-        done_cv_.wait(lk, finished);
-    else if (!done_cv_.wait_for(lk, timeout, finished))
-        return false;
-    if (error_) std::rethrow_exception(error_);
-    return true;
-}
-
 std::vector<at::Tensor> WorkMCCL::result() { return outputs_; }
 
 c10::intrusive_ptr<c10::ivalue::Future> WorkMCCL::getFuture() { return future_; }
-
-// First caller wins; later finish()/finishWithException() calls are no-ops.
-bool WorkMCCL::complete(std::exception_ptr error) {
-    std::lock_guard<std::mutex> lk(mu_);
-    if (done_.load(std::memory_order_acquire)) return false;
-    error_ = error;
-    done_.store(true, std::memory_order_release);
-    return true;
-}
-
-void WorkMCCL::finish() {
-    if (sync_) {
-        try {
-            sync_();
-        } catch (...) {
-            finishWithException(std::current_exception());
-            return;
-        }
-    }
-    if (!complete(nullptr)) return;
-    if (future_ && !future_->completed()) future_->markCompleted(c10::IValue(outputs_));
-    done_cv_.notify_all();
-}
-
-void WorkMCCL::finishWithException(std::exception_ptr error) {
-    if (!complete(error)) return;
-    if (future_ && !future_->completed()) future_->setError(error);
-    done_cv_.notify_all();
-}
 
 }  // namespace mccl

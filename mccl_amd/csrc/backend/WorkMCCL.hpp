@@ -1,10 +1,13 @@
 // WorkMCCL.hpp -- completion object of one collective (c10d::Work).
 //
-// Contract of the reference's csrc/backend/WorkMCCL.{hpp,cpp}: created when the
-// collective is issued; finish() runs an optional sync callback (which drains
-// the reduce queue) and then completes the Work and its Future with the output
-// tensors; finishWithException() completes both with the error; wait() blocks
-// until then, returns false on timeout and rethrows the stored error.
+// Observable contract of the reference's csrc/backend/WorkMCCL.{hpp,cpp}: the
+// object exists from the moment the collective is issued; finish() first runs
+// an optional callback (which drains the reduce queue) and then settles the
+// Work and its Future with the output tensors; finishWithException() settles
+// both with the error; wait() blocks until then, returns false when the
+// timeout passes first and rethrows a stored error.
+//
+// One state variable under one mutex: Pending -> Succeeded | Failed, once.
 #pragma once
 
 #include <torch/csrc/distributed/c10d/Types.hpp>
@@ -12,7 +15,6 @@
 
 #include <ATen/ATen.h>
 
-#include <atomic>
 #include <chrono>
 #include <condition_variable>
 #include <exception>
@@ -27,27 +29,33 @@ public:
     WorkMCCL(c10d::OpType op, std::vector<at::Tensor> outputs, const char* title = "mccl:work");
     ~WorkMCCL() override;
 
+    // -- what the issuing side calls (the engine thread, or the caller's thread for allreduce)
+    void setSyncCallback(std::function<void()> before_done) { before_done_ = std::move(before_done); }
+    void finish();
+    void finishWithException(std::exception_ptr error);
+
+    // -- c10d::Work
+    bool wait(std::chrono::milliseconds timeout = kNoTimeout) override;
     bool isCompleted() override;
     bool isSuccess() const override;
     std::exception_ptr exception() const override;
-    bool wait(std::chrono::milliseconds timeout = kNoTimeout) override;
     std::vector<at::Tensor> result() override;
     c10::intrusive_ptr<c10::ivalue::Future> getFuture() override;
 
-    void finish();
-    void finishWithException(std::exception_ptr error);
-    void setSyncCallback(std::function<void()> cb) { sync_ = std::move(cb); }
-
 private:
-    bool complete(std::exception_ptr error);
+    enum class State { Pending, Succeeded, Failed };
 
-    mutable std::mutex mu_;
-    std::condition_variable done_cv_;
-    std::atomic<bool> done_{false};
-    std::exception_ptr error_;
+    // First call wins; later ones do nothing.
+    void settle(std::exception_ptr error);
+
     std::vector<at::Tensor> outputs_;
     c10::intrusive_ptr<c10::ivalue::Future> future_;
-    std::function<void()> sync_;
+    std::function<void()> before_done_;
+
+    mutable std::mutex mu_;
+    std::condition_variable settled_cv_;
+    State state_ = State::Pending;
+    std::exception_ptr error_;
 };
 
 }  // namespace mccl
