@@ -489,12 +489,17 @@ def test_recv_times_out_when_nothing_was_sent(CX):
             msgs[1] = "sent"
         else:
             t = torch.empty(4, device="cuda")
-            pg.recv([t], 1, 3).wait()
+            for attempt in range(10):          # each attempt waits up to the group's 2 s
+                try:
+                    pg.recv([t], 1, 3).wait()
+                    break
+                except RuntimeError:
+                    continue
             msgs.append(t.cpu().tolist())
 
     ts = [threading.Thread(target=body, args=(r,)) for r in range(2)]
     [t.start() for t in ts]
-    [t.join(30) for t in ts]
+    [t.join(60) for t in ts]
     assert not any(t.is_alive() for t in ts)
     assert "Timeout" in msgs[0] and "nothing arrived from rank 1" in msgs[0]
     assert msgs[2] == [9.0] * 4
