@@ -91,6 +91,33 @@ def test_init_process_group_world_one(CX):
         dist.destroy_process_group()
 
 
+def test_distributed_data_parallel_over_the_backend_world_one(CX):
+    """torch's DistributedDataParallel on top of backend "mccl" (the reference's
+    tests/test_ddp.py:70-95 shape: a Linear layer, SGD, a few steps): parameter
+    broadcast, bucket allreduce through Work/Future, and the same weights as plain training."""
+    from torch.nn.parallel import DistributedDataParallel as DDP
+    if dist.is_initialized():
+        dist.destroy_process_group()
+    dist.init_process_group(backend="mccl", store=dist.HashStore(), rank=0, world_size=1, timeout=TIMEOUT)
+    try:
+        torch.manual_seed(42)
+        plain = torch.nn.Linear(16, 1, bias=False).cuda()
+        wrapped = DDP(torch.nn.Linear(16, 1, bias=False).cuda())
+        wrapped.module.load_state_dict(plain.state_dict())
+        opt_a = torch.optim.SGD(plain.parameters(), lr=0.01)
+        opt_b = torch.optim.SGD(wrapped.parameters(), lr=0.01)
+        x = torch.randn(32, 16, device="cuda")
+        y = torch.randn(32, 1, device="cuda")
+        for _ in range(5):
+            for model, opt in ((plain, opt_a), (wrapped, opt_b)):
+                opt.zero_grad()
+                torch.nn.functional.mse_loss(model(x), y).backward()
+                opt.step()
+        assert torch.equal(plain.weight, wrapped.module.weight)
+    finally:
+        dist.destroy_process_group()
+
+
 # ---- N ranks in one process -----------------------------------------------------------
 
 @pytest.mark.parametrize("world", [2, 3, 4])
