@@ -98,6 +98,10 @@ MCCLX_API void* mcclx_queue_stream(mcclx_ctx* ctx);
 /* Number of compute units of the context's device (sizing of persistent grids). */
 MCCLX_API int mcclx_device_cus(mcclx_ctx* ctx);
 
+/* Diagnostic: kernel launches this context has issued so far (recorded ones
+ * count when they are recorded, not when a graph replays them). */
+MCCLX_API uint64_t mcclx_launch_count(mcclx_ctx* ctx);
+
 /* ---- the reference's four kernel entry points, one to one ------------------- */
 
 /* dst[i] = dst[i] (op) src[i].  Replaces metal_reduce_op_view

@@ -64,6 +64,7 @@ SIGNATURES = {
     "mcclx_destroy": (_i, [_vp]),
     "mcclx_queue_stream": (_vp, [_vp]),
     "mcclx_device_cus": (_i, [_vp]),
+    "mcclx_launch_count": (_u64, [_vp]),
     "mcclx_reduce": (_i, [_vp, _vp, _vp, _i, _u64, _i]),
     "mcclx_scale": (_i, [_vp, _vp, _i, _u64, _d, _i]),
     "mcclx_accumulate_scale": (_i, [_vp, _vp, _vp, _i, _u64, _d]),

@@ -8,6 +8,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <atomic>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -71,6 +72,7 @@ struct mcclx_ctx {
     bool own_stream = false;
     int cus = 0;
     uint32_t max_blocks = 0;
+    std::atomic<uint64_t> launches{0};  // kernel launches issued (diagnostic)
     uint32_t few_max = mcclx::kFewSegs;  // segments up to which descriptors travel in the kernel arguments
     bool validate = false;
     bool batch_active = false;
@@ -391,6 +393,7 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
         lp.few = &a;
         hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
         if (e != hipSuccess) return launch_error(e, key);
+        ++ctx->launches;
         return MCCLX_OK;
     }
 
@@ -438,6 +441,7 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
     lp.table = &t;
     hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
     if (e != hipSuccess) return launch_error(e, key);
+    ++ctx->launches;
     return table_launched(ctx, slot);
 }
 
@@ -538,6 +542,7 @@ int mcclx_destroy(mcclx_ctx* ctx) {
 
 void* mcclx_queue_stream(mcclx_ctx* ctx) { return ctx ? (void*)ctx->stream : nullptr; }
 int mcclx_device_cus(mcclx_ctx* ctx) { return ctx ? ctx->cus : 0; }
+uint64_t mcclx_launch_count(mcclx_ctx* ctx) { return ctx ? ctx->launches.load() : 0; }
 
 int mcclx_fold(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* seg) {
     return fold_impl(ctx, plan, seg, 1);
@@ -616,6 +621,7 @@ int mcclx_copy(mcclx_ctx* ctx, void* dst, const void* src, uint64_t nbytes) {
     DeviceGuard guard(ctx->device);
     hipError_t e = mcclx::launch_copy(ctx->stream, dst, src, nbytes, ctx->max_blocks);
     if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "copy launch failed: %s", hipGetErrorString(e));
+    ++ctx->launches;
     return MCCLX_OK;
 }
 
@@ -690,6 +696,7 @@ int mcclx_copy_batched(mcclx_ctx* ctx, const mcclx_copy_desc* descs, uint32_t n)
     int align = (both % 4 == 0) ? 4 : (both % 2 == 0) ? 2 : 1;
     hipError_t e = mcclx::launch_copy_many(ctx->stream, t, align, ctx->max_blocks);
     if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "copy_batched launch failed: %s", hipGetErrorString(e));
+    ++ctx->launches;
     return table_launched(ctx, slot);
 }
 

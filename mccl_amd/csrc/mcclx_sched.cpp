@@ -207,15 +207,24 @@ struct Phases {
     std::vector<mcclx_copy_desc> copies;
 };
 
+// MIN / MAX / PRODUCT over the wire codec: the fold kernels mix fp32 and bf16
+// operands for sums only, so for these ops every rank encodes its WHOLE tensor
+// (the owner's chunk too), the fold runs on bf16 operands alone, in place over
+// the owner's wire copy, and every rank -- the owner included -- casts the
+// result back.  Same arithmetic as the reference (cast, reduce in bf16, cast
+// back: ProcessGroupMCCL.cpp:131-132, 179-183), in three launches.
+bool all_on_wire(const mcclx_replay* r) { return r->op != MCCLX_SUM && r->op != MCCLX_AVG; }
+
 void plan_phases(const mcclx_replay* r, const Layout& L, Phases& ph) {
     if (ph.planned) return;
     ph.planned = true;
     ph.fold = base_plan(r, L, r->world);
-    if (r->algo == MCCLX_ALGO_TREE) {
-        ph.fold.topo = MCCLX_TOPO_BINOMIAL;
-        if (L.wire) ph.fold.io = MCCLX_IO_OWN_FIRST_F32;
-    } else if (L.wire) {
-        ph.fold.io = r->algo == MCCLX_ALGO_RING ? MCCLX_IO_OWN_LAST_F32 : MCCLX_IO_OWN_FIRST_F32;
+    if (r->algo == MCCLX_ALGO_TREE) ph.fold.topo = MCCLX_TOPO_BINOMIAL;
+    if (L.wire && !all_on_wire(r)) {  // the owner's operand is read as fp32 and encoded in registers
+        if (r->algo == MCCLX_ALGO_TREE)
+            ph.fold.io = MCCLX_IO_OWN_FIRST_F32;
+        else
+            ph.fold.io = r->algo == MCCLX_ALGO_RING ? MCCLX_IO_OWN_LAST_F32 : MCCLX_IO_OWN_FIRST_F32;
     }
     ph.enc = base_plan(r, L, 1);  // fp32 -> bf16 of what travels
     ph.enc.io = MCCLX_IO_OWN_FIRST_F32;
@@ -234,11 +243,12 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
     mcclx_seg z;
     memset(&z, 0, sizeof z);
 
+    const bool bf16_only = L.wire && all_on_wire(r);
     if (r->algo == MCCLX_ALGO_TREE) {
         // allreduce_tree: rank 0 ends with the binomial combination of all
         // tensors (AllreduceAlgos.cpp:100-114), everyone else receives a copy.
         if (L.wire)
-            for (int q = 1; q < N; ++q) {  // ranks 1.. encode: their tensors travel
+            for (int q = bf16_only ? 0 : 1; q < N; ++q) {  // ranks 1.. encode: their tensors travel
                 mcclx_seg s = z;
                 s.wire_out = wire_of(q);
                 s.in[0] = r->tensors[q];
@@ -246,13 +256,18 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
                 ph.enc_segs.push_back(s);
             }
         mcclx_seg s = z;
-        s.out = r->tensors[0];
         s.count = r->numel;
-        s.in[0] = r->tensors[0];
-        for (int q = 1; q < N; ++q) s.in[q] = L.wire ? wire_of(q) : r->tensors[q];
-        if (L.wire) s.wire_out = wire_of(0);
+        if (bf16_only) {
+            s.out = wire_of(0);
+            for (int q = 0; q < N; ++q) s.in[q] = wire_of(q);
+        } else {
+            s.out = r->tensors[0];
+            s.in[0] = r->tensors[0];
+            for (int q = 1; q < N; ++q) s.in[q] = L.wire ? wire_of(q) : r->tensors[q];
+            if (L.wire) s.wire_out = wire_of(0);
+        }
         ph.fold_segs.push_back(s);
-        for (int q = 1; q < N; ++q) {
+        for (int q = bf16_only ? 0 : 1; q < N; ++q) {
             if (L.wire) {  // broadcast of the bf16 result + the final cast on every rank
                 mcclx_seg g = z;
                 g.out = r->tensors[q];
@@ -281,7 +296,7 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
     if (L.wire)  // every rank encodes what it sends: all chunks except the one it owns
         for (int q = 0; q < N; ++q)
             for (int ch = 0; ch < N; ++ch) {
-                if (owner_of(ch) == q || c[ch].elem_count == 0) continue;
+                if ((owner_of(ch) == q && !bf16_only) || c[ch].elem_count == 0) continue;
                 mcclx_seg s = z;
                 s.wire_out = at(wire_of(q), (uint64_t)c[ch].elem_start * 2);
                 s.in[0] = at(r->tensors[q], (uint64_t)c[ch].elem_start * 4);
@@ -294,11 +309,15 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
         int o = owner_of(ch);
         mcclx_seg s = z;
         s.count = (uint64_t)c[ch].elem_count;
-        s.out = at(r->tensors[o], (uint64_t)c[ch].elem_start * ts);
-        if (L.wire) s.wire_out = at(wire_of(o), (uint64_t)c[ch].elem_start * 2);
+        if (bf16_only) {
+            s.out = at(wire_of(o), (uint64_t)c[ch].elem_start * 2);
+        } else {
+            s.out = at(r->tensors[o], (uint64_t)c[ch].elem_start * ts);
+            if (L.wire) s.wire_out = at(wire_of(o), (uint64_t)c[ch].elem_start * 2);
+        }
         for (int j = 0; j < N; ++j) {
             int q = order_of(ch, j);
-            if (L.wire && q != o)
+            if (L.wire && (q != o || bf16_only))
                 s.in[j] = at(wire_of(q), (uint64_t)c[ch].elem_start * es);
             else
                 s.in[j] = at(r->tensors[q], (uint64_t)c[ch].elem_start * ts);
@@ -313,7 +332,7 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
         if (c[ch].elem_count == 0) continue;
         int o = owner_of(ch);
         for (int q = 0; q < N; ++q) {
-            if (q == o) continue;
+            if (q == o && !bf16_only) continue;
             if (L.wire) {
                 mcclx_seg s = z;
                 s.out = at(r->tensors[q], (uint64_t)c[ch].elem_start * 4);
@@ -363,11 +382,7 @@ int check_replay(mcclx_ctx* ctx, const mcclx_replay* r, bool* fused, bool* nothi
         if (!r->tensors[i]) return bad("replay: null tensor");
     Layout L = layout_of(r);
     if (L.total > 0 && (!r->workspace || r->workspace_bytes < L.total)) return bad("workspace too small");
-    bool f = r->mode == MCCLX_REPLAY_FUSED && r->world <= MCCLX_MAX_INPUTS;
-    // The wire codec mixes fp32 and bf16 operands, which only the SUM fold
-    // handles; MIN / MAX / PRODUCT over the wire run the stepwise schedule.
-    if (f && L.wire && r->op != MCCLX_SUM && r->op != MCCLX_AVG) f = false;
-    *fused = f;
+    *fused = r->mode == MCCLX_REPLAY_FUSED && r->world <= MCCLX_MAX_INPUTS;
     return MCCLX_OK;
 }
 

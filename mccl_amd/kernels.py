@@ -178,6 +178,10 @@ class ReduceQueue:
         arr = (L.Seg * len(segs))(*segs)
         L.check(L.lib().mcclx_fold_batched(self.handle, C.byref(plan), arr, len(segs)))
 
+    def launch_count(self) -> int:
+        """Kernel launches issued on this queue so far (diagnostic)."""
+        return int(L.lib().mcclx_launch_count(self.handle))
+
     def copy(self, dst_ptr: int, src_ptr: int, nbytes: int) -> None:
         L.check(L.lib().mcclx_copy(self.handle, C.c_void_p(dst_ptr), C.c_void_p(src_ptr), nbytes))
 

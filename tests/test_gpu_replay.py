@@ -248,3 +248,30 @@ def test_copy_batched_many_small_and_a_few_large(K, U):
         q.copy_batched(triples)
         q.drain()
         assert np.array_equal(dst.cpu().numpy(), want), sizes[:5]
+
+
+def test_launch_counts_of_the_fused_schedules(H, K, U):
+    """What "fused" means in launches: butterfly over the wire = encode + fold + cast (3), for any
+    reduce op; without the wire 1 fold + the allgather copies; a list of 200 tree messages = 1 fold
+    + 1 copy launch; the stepwise replay of the same butterfly issues the reference's sequence."""
+    from mccl_amd import _lib as L
+    q = K._q(None)
+    world, n = 3, 300_000
+    rng = np.random.default_rng(8)
+
+    def launches(fn):
+        before = q.launch_count()
+        fn()
+        return q.launch_count() - before
+
+    mk = lambda: [U.to_dev(U.rand_values(rng, n, F32), F32) for _ in range(world)]
+    for op in ("avg", "min", "max", "product"):
+        t = mk()
+        assert launches(lambda: H.allreduce_replay(t, op, BUTTERFLY, wire_bf16=True, mode=FUSED)) == 3, op
+    t = mk()
+    assert launches(lambda: H.allreduce_replay(t, "sum", BUTTERFLY, mode=FUSED)) == 1 + 1   # 6 copies of 400 KB: one launch
+    t = mk()
+    stepwise = launches(lambda: H.allreduce_replay(t, "avg", BUTTERFLY, wire_bf16=True, mode=STEPWISE))
+    assert stepwise >= 3 + 2 * 3 * 2 + 3 + 3       # encodes, (copy + reduce) per peer and rank, scales, ..., decodes
+    groups = [[U.to_dev(U.rand_values(rng, 5000 + 7 * i, F32), F32) for _ in range(world)] for i in range(200)]
+    assert launches(lambda: H.allreduce_replay_many(groups, "sum", TREE)) == 2
