@@ -200,10 +200,16 @@ mcclx_plan base_plan(const mcclx_replay* r, const Layout& L, int k) {
 // The launches of one or more fused allreduces that share a plan, gathered phase
 // by phase: what every rank encodes for the wire, the folds, the casts on
 // arrival, and the plain copies of the allgather leg.  Each phase is one launch.
+struct FoldPass {
+    mcclx_plan plan;
+    std::vector<mcclx_seg> segs;
+};
+
 struct Phases {
     bool planned = false;
-    mcclx_plan enc, fold, dec;
-    std::vector<mcclx_seg> enc_segs, fold_segs, dec_segs;
+    mcclx_plan enc, dec;
+    std::vector<mcclx_seg> enc_segs, dec_segs;
+    std::vector<FoldPass> folds;  // one pass, or a chain of passes when the world is wider than one fold
     std::vector<mcclx_copy_desc> copies;
 };
 
@@ -213,18 +219,47 @@ struct Phases {
 // the owner's wire copy, and every rank -- the owner included -- casts the
 // result back.  Same arithmetic as the reference (cast, reduce in bf16, cast
 // back: ProcessGroupMCCL.cpp:131-132, 179-183), in three launches.
-bool all_on_wire(const mcclx_replay* r) { return r->op != MCCLX_SUM && r->op != MCCLX_AVG; }
+// The same holds for a world wider than one fold (see chain_lengths).
+bool all_on_wire(const mcclx_replay* r) {
+    return (r->op != MCCLX_SUM && r->op != MCCLX_AVG) || r->world > MCCLX_MAX_INPUTS;
+}
+
+// A fold takes MCCLX_MAX_INPUTS operands.  A wider world is folded by a chain
+// of passes over same-dtype buffers: the first takes 8 operands, every later
+// one the partial result plus up to 7 more, in the schedule's own order -- a
+// left fold cut into pieces, so rounding happens exactly where the one-pass
+// fold (and the reference's step-by-step loop) has it.  The scale goes with
+// the last pass.
+std::vector<int> chain_lengths(int world) {
+    std::vector<int> ks;
+    int left = world;
+    ks.push_back(left < MCCLX_MAX_INPUTS ? left : MCCLX_MAX_INPUTS);
+    left -= ks.back();
+    while (left > 0) {
+        int more = left < MCCLX_MAX_INPUTS - 1 ? left : MCCLX_MAX_INPUTS - 1;
+        ks.push_back(more + 1);  // + the partial result
+        left -= more;
+    }
+    return ks;
+}
 
 void plan_phases(const mcclx_replay* r, const Layout& L, Phases& ph) {
     if (ph.planned) return;
     ph.planned = true;
-    ph.fold = base_plan(r, L, r->world);
-    if (r->algo == MCCLX_ALGO_TREE) ph.fold.topo = MCCLX_TOPO_BINOMIAL;
+    const std::vector<int> ks = chain_lengths(r->world);
+    ph.folds.resize(ks.size());
+    for (size_t p = 0; p < ks.size(); ++p) {
+        mcclx_plan& f = ph.folds[p].plan;
+        f = base_plan(r, L, ks[p]);
+        if (p + 1 < ks.size()) f.scale_mode = MCCLX_SCALE_NONE;  // only the last pass scales
+    }
+    mcclx_plan& fold = ph.folds[0].plan;
+    if (r->algo == MCCLX_ALGO_TREE) fold.topo = MCCLX_TOPO_BINOMIAL;
     if (L.wire && !all_on_wire(r)) {  // the owner's operand is read as fp32 and encoded in registers
         if (r->algo == MCCLX_ALGO_TREE)
-            ph.fold.io = MCCLX_IO_OWN_FIRST_F32;
+            fold.io = MCCLX_IO_OWN_FIRST_F32;
         else
-            ph.fold.io = r->algo == MCCLX_ALGO_RING ? MCCLX_IO_OWN_LAST_F32 : MCCLX_IO_OWN_FIRST_F32;
+            fold.io = r->algo == MCCLX_ALGO_RING ? MCCLX_IO_OWN_LAST_F32 : MCCLX_IO_OWN_FIRST_F32;
     }
     ph.enc = base_plan(r, L, 1);  // fp32 -> bf16 of what travels
     ph.enc.io = MCCLX_IO_OWN_FIRST_F32;
@@ -266,7 +301,7 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
             for (int q = 1; q < N; ++q) s.in[q] = L.wire ? wire_of(q) : r->tensors[q];
             if (L.wire) s.wire_out = wire_of(0);
         }
-        ph.fold_segs.push_back(s);
+        ph.folds[0].segs.push_back(s);
         for (int q = bf16_only ? 0 : 1; q < N; ++q) {
             if (L.wire) {  // broadcast of the bf16 result + the final cast on every rank
                 mcclx_seg g = z;
@@ -307,22 +342,41 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
     for (int ch = 0; ch < N; ++ch) {
         if (c[ch].elem_count == 0) continue;
         int o = owner_of(ch);
-        mcclx_seg s = z;
-        s.count = (uint64_t)c[ch].elem_count;
-        if (bf16_only) {
-            s.out = at(wire_of(o), (uint64_t)c[ch].elem_start * 2);
-        } else {
-            s.out = at(r->tensors[o], (uint64_t)c[ch].elem_start * ts);
-            if (L.wire) s.wire_out = at(wire_of(o), (uint64_t)c[ch].elem_start * 2);
-        }
+        // operands in schedule order, and where the result goes
+        std::vector<const void*> ops((size_t)N);
         for (int j = 0; j < N; ++j) {
             int q = order_of(ch, j);
             if (L.wire && (q != o || bf16_only))
-                s.in[j] = at(wire_of(q), (uint64_t)c[ch].elem_start * es);
+                ops[(size_t)j] = at(wire_of(q), (uint64_t)c[ch].elem_start * es);
             else
-                s.in[j] = at(r->tensors[q], (uint64_t)c[ch].elem_start * ts);
+                ops[(size_t)j] = at(r->tensors[q], (uint64_t)c[ch].elem_start * ts);
         }
-        ph.fold_segs.push_back(s);
+        void* dest = bf16_only ? (void*)at(wire_of(o), (uint64_t)c[ch].elem_start * 2)
+                               : (void*)at(r->tensors[o], (uint64_t)c[ch].elem_start * ts);
+        if (ph.folds.size() == 1) {
+            mcclx_seg s = z;
+            s.count = (uint64_t)c[ch].elem_count;
+            s.out = dest;
+            if (L.wire && !bf16_only) s.wire_out = at(wire_of(o), (uint64_t)c[ch].elem_start * 2);
+            for (int j = 0; j < N; ++j) s.in[j] = ops[(size_t)j];
+            ph.folds[0].segs.push_back(s);
+            continue;
+        }
+        // A chain.  Butterfly's first operand is the owner's own chunk, so the partial
+        // result can live in `dest` from the first pass on; ring's owner comes last, so
+        // the partial result waits in the owner's recv scratch until the last pass.
+        void* partial = ring ? (void*)at(r->workspace, L.scratch_off + (uint64_t)o * L.scratch_stride) : dest;
+        int next = 0;
+        for (size_t p = 0; p < ph.folds.size(); ++p) {
+            const int k = ph.folds[p].plan.k;
+            mcclx_seg s = z;
+            s.count = (uint64_t)c[ch].elem_count;
+            int j = 0;
+            if (p > 0) s.in[j++] = partial;
+            while (j < k) s.in[j++] = ops[(size_t)next++];
+            s.out = (p + 1 == ph.folds.size()) ? dest : partial;
+            ph.folds[p].segs.push_back(s);
+        }
     }
 
     // allgather leg (AllreduceAlgos.cpp:77-86,185-200): every other rank gets
@@ -351,8 +405,8 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
 int issue_phases(mcclx_ctx* ctx, Phases& ph) {
     if (!ph.enc_segs.empty())
         TRY(mcclx_fold_batched(ctx, &ph.enc, ph.enc_segs.data(), (uint32_t)ph.enc_segs.size()));
-    if (!ph.fold_segs.empty())
-        TRY(mcclx_fold_batched(ctx, &ph.fold, ph.fold_segs.data(), (uint32_t)ph.fold_segs.size()));
+    for (FoldPass& f : ph.folds)
+        if (!f.segs.empty()) TRY(mcclx_fold_batched(ctx, &f.plan, f.segs.data(), (uint32_t)f.segs.size()));
     if (!ph.dec_segs.empty())
         TRY(mcclx_fold_batched(ctx, &ph.dec, ph.dec_segs.data(), (uint32_t)ph.dec_segs.size()));
     if (!ph.copies.empty()) TRY(mcclx_copy_batched(ctx, ph.copies.data(), (uint32_t)ph.copies.size()));
@@ -382,7 +436,8 @@ int check_replay(mcclx_ctx* ctx, const mcclx_replay* r, bool* fused, bool* nothi
         if (!r->tensors[i]) return bad("replay: null tensor");
     Layout L = layout_of(r);
     if (L.total > 0 && (!r->workspace || r->workspace_bytes < L.total)) return bad("workspace too small");
-    *fused = r->mode == MCCLX_REPLAY_FUSED && r->world <= MCCLX_MAX_INPUTS;
+    // the binomial tree of more than MCCLX_MAX_INPUTS ranks does not cut into a chain of folds
+    *fused = r->mode == MCCLX_REPLAY_FUSED && (r->world <= MCCLX_MAX_INPUTS || r->algo != MCCLX_ALGO_TREE);
     return MCCLX_OK;
 }
 
@@ -483,8 +538,7 @@ int mcclx_reduce_scatter_shares(mcclx_ctx* ctx, int world, void* const* outs,
     if (world == 1) return mcclx_copy(ctx, outs[0], share(0, 0), cb);  // ProcessGroupMCCL.cpp:333-337
     // MIN / MAX / PRODUCT and fp16 round after every step by definition
     bool step_only = (op != MCCLX_SUM && op != MCCLX_AVG) || dtype == MCCLX_F16;
-    bool fused = mode == MCCLX_REPLAY_FUSED && world <= MCCLX_MAX_INPUTS;
-    if (!fused) {
+    if (mode != MCCLX_REPLAY_FUSED) {
         for (int r = 0; r < world; ++r) {  // :357, :378-386
             TRY(mcclx_copy(ctx, outs[r], share(r, r), cb));
             for (int p = 0; p < world; ++p)
@@ -494,27 +548,41 @@ int mcclx_reduce_scatter_shares(mcclx_ctx* ctx, int world, void* const* outs,
         }
         return MCCLX_OK;
     }
+    // One fold per rank; a world wider than one fold is cut into a chain of passes
+    // (chain_lengths), the partial result waiting in the rank's output between them.
+    // fp32 accumulation (ACC_F32) has a meaning inside one fold only: a chain rounds
+    // where it is cut, so it runs with per-step rounding.
+    const std::vector<int> ks = chain_lengths(world);
     mcclx_plan p;
     memset(&p, 0, sizeof p);
     p.dtype = dtype;
     p.io = MCCLX_IO_PURE;
-    p.k = world;
     p.topo = MCCLX_TOPO_FOLD;
     p.op = op;
-    p.acc = step_only ? MCCLX_ACC_STEP : acc;
-    p.scale_mode = (op == MCCLX_AVG) ? MCCLX_SCALE_TENSOR : MCCLX_SCALE_NONE;  // metal_scale_inplace
+    p.acc = (step_only || ks.size() > 1) ? MCCLX_ACC_STEP : acc;
     p.scale = 1.0 / (double)world;
-    std::vector<mcclx_seg> segs((size_t)world);
-    for (int r = 0; r < world; ++r) {
-        memset(&segs[r], 0, sizeof(mcclx_seg));
-        segs[r].out = outs[r];
-        segs[r].count = chunk_numel;
-        segs[r].in[0] = share(r, r);  // own share first (:357)
-        int j = 1;
-        for (int q = 0; q < world; ++q)
-            if (q != r) segs[r].in[j++] = share(r, q);  // ascending peers (:379-383)
+    std::vector<int> next((size_t)world, 0);  // per rank: operands consumed so far
+    auto operand = [&](int r, int j) {        // own share first (:357), then ascending peers (:379-383)
+        if (j == 0) return share(r, r);
+        return share(r, (j - 1 < r) ? j - 1 : j);
+    };
+    for (size_t pass = 0; pass < ks.size(); ++pass) {
+        p.k = ks[pass];
+        const bool last = pass + 1 == ks.size();
+        p.scale_mode = (last && op == MCCLX_AVG) ? MCCLX_SCALE_TENSOR : MCCLX_SCALE_NONE;  // metal_scale_inplace
+        std::vector<mcclx_seg> segs((size_t)world);
+        for (int r = 0; r < world; ++r) {
+            mcclx_seg& g = segs[(size_t)r];
+            memset(&g, 0, sizeof g);
+            g.out = outs[r];
+            g.count = chunk_numel;
+            int j = 0;
+            if (pass > 0) g.in[j++] = outs[r];
+            while (j < p.k) g.in[j++] = operand(r, next[(size_t)r]++);
+        }
+        TRY(mcclx_fold_batched(ctx, &p, segs.data(), (uint32_t)segs.size()));
     }
-    return mcclx_fold_batched(ctx, &p, segs.data(), (uint32_t)segs.size());
+    return MCCLX_OK;
 }
 
 int mcclx_reduce_scatter_replay(mcclx_ctx* ctx, int world, void* const* outs,

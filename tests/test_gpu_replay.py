@@ -77,9 +77,15 @@ def test_allreduce_other_ops_and_fp16(H, U, algo, op, mode):
 
 
 @pytest.mark.parametrize("algo", [RING, TREE, BUTTERFLY])
-def test_wide_world_falls_back_to_stepwise(H, U, algo):
+def test_worlds_wider_than_one_fold(H, U, algo):
+    """More ranks than one fold takes operands: ring and butterfly chain folds (8 operands, then
+    the partial result + 7 more, ...), the tree runs the stepwise schedule; all bit-exact."""
     run_case(H, U, algo, 11, F32, SUM, True, FUSED, 2003, seed=11)
     run_case(H, U, algo, 16, BF16, AVG, False, FUSED, 2003, seed=16)
+    run_case(H, U, algo, 9, F32, AVG, False, FUSED, 40009, seed=9, specials=True)
+    run_case(H, U, algo, 23, F32, AVG, True, FUSED, 5003, seed=23, specials=True)
+    run_case(H, U, algo, 10, BF16, MAX, False, FUSED, 3001, seed=10)
+    run_case(H, U, algo, 12, F32, PRODUCT, True, FUSED, 3001, seed=12)
 
 
 def test_tree_with_fewer_elements_than_ranks(H, U):  # ProcessGroupMCCL.cpp:143-145 -> tree
@@ -138,7 +144,7 @@ def test_env_semantics(H, U, monkeypatch):
     U.assert_same_bits(d[0], want[0], F32, "no wire")
 
 
-@pytest.mark.parametrize("world", [2, 3, 8, 10])
+@pytest.mark.parametrize("world", [2, 3, 8, 10, 17])
 @pytest.mark.parametrize("dtype", [F32, BF16, F16])
 @pytest.mark.parametrize("mode", [STEPWISE, FUSED])
 def test_reduce_scatter_allgather(H, U, world, dtype, mode):
@@ -275,3 +281,5 @@ def test_launch_counts_of_the_fused_schedules(H, K, U):
     assert stepwise >= 3 + 2 * 3 * 2 + 3 + 3       # encodes, (copy + reduce) per peer and rank, scales, ..., decodes
     groups = [[U.to_dev(U.rand_values(rng, 5000 + 7 * i, F32), F32) for _ in range(world)] for i in range(200)]
     assert launches(lambda: H.allreduce_replay_many(groups, "sum", TREE)) == 2
+    wide = [U.to_dev(U.rand_values(rng, n, F32), F32) for _ in range(16)]     # 16 ranks: folds of 8, 8 and 2 operands
+    assert launches(lambda: H.allreduce_replay(wide, "avg", RING, wire_bf16=True, mode=FUSED)) == 1 + 3 + 1
