@@ -418,7 +418,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
             rp.acc = MCCLX_ACC_STEP;
             rp.numel = all[0].numel[i];
             rp.tensors = ptrs[i].data();
-            // size for the stepwise fallback too (a tree of more than 8 ranks)
+            // size for the stepwise fallback too (a tree of more than 64 ranks)
             mcclx_replay st = rp;
             st.mode = MCCLX_REPLAY_STEPWISE;
             need[i] = (std::max(mcclx_replay_workspace_bytes(&rp), mcclx_replay_workspace_bytes(&st)) + 255) / 256 * 256;

@@ -246,6 +246,29 @@ std::vector<int> chain_lengths(int world) {
 void plan_phases(const mcclx_replay* r, const Layout& L, Phases& ph) {
     if (ph.planned) return;
     ph.planned = true;
+    if (r->algo == MCCLX_ALGO_TREE && r->world > MCCLX_MAX_INPUTS) {
+        // The binomial tree of up to 64 ranks is a binomial tree of binomial trees:
+        // masks 1, 2, 4 combine each block of 8 consecutive ranks into its first
+        // rank, masks 8, 16, 32 combine the blocks' first ranks the same way
+        // (AllreduceAlgos.cpp:100-114).  Pass 0 folds the full blocks, pass 1 the
+        // last, shorter block, pass 2 the block results into rank 0 (and scales).
+        const int blocks = (r->world + MCCLX_MAX_INPUTS - 1) / MCCLX_MAX_INPUTS;
+        const int last = r->world - (blocks - 1) * MCCLX_MAX_INPUTS;
+        ph.folds.resize(3);
+        const int ks3[3] = {MCCLX_MAX_INPUTS, last, blocks};
+        for (int p = 0; p < 3; ++p) {
+            ph.folds[(size_t)p].plan = base_plan(r, L, ks3[p]);
+            ph.folds[(size_t)p].plan.topo = MCCLX_TOPO_BINOMIAL;
+            if (p < 2) ph.folds[(size_t)p].plan.scale_mode = MCCLX_SCALE_NONE;
+        }
+        ph.enc = base_plan(r, L, 1);
+        ph.enc.io = MCCLX_IO_OWN_FIRST_F32;
+        ph.enc.op = MCCLX_SUM;
+        ph.enc.scale_mode = MCCLX_SCALE_NONE;
+        ph.dec = ph.enc;
+        ph.dec.io = MCCLX_IO_OUT_F32;
+        return;
+    }
     const std::vector<int> ks = chain_lengths(r->world);
     ph.folds.resize(ks.size());
     for (size_t p = 0; p < ks.size(); ++p) {
@@ -290,6 +313,37 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
                 s.count = r->numel;
                 ph.enc_segs.push_back(s);
             }
+        if (N > MCCLX_MAX_INPUTS) {  // blocks of 8 ranks, then the blocks' first ranks (see plan_phases)
+            auto buf = [&](int q) -> void* { return bf16_only ? wire_of(q) : r->tensors[q]; };
+            const int blocks = (N + MCCLX_MAX_INPUTS - 1) / MCCLX_MAX_INPUTS;
+            mcclx_seg top = z;
+            top.count = r->numel;
+            top.out = buf(0);
+            for (int b = 0; b < blocks; ++b) {
+                const int first = b * MCCLX_MAX_INPUTS;
+                const int kb = (N - first < MCCLX_MAX_INPUTS) ? N - first : MCCLX_MAX_INPUTS;
+                top.in[b] = buf(first);
+                if (kb < 2) continue;  // a block of one rank is its own result
+                mcclx_seg g = z;
+                g.count = r->numel;
+                g.out = buf(first);    // intermediate ranks' buffers hold partial sums, as in the reference
+                for (int j = 0; j < kb; ++j) g.in[j] = buf(first + j);
+                ph.folds[kb == MCCLX_MAX_INPUTS ? 0 : 1].segs.push_back(g);
+            }
+            ph.folds[2].segs.push_back(top);
+            for (int q = bf16_only ? 0 : 1; q < N; ++q) {
+                if (L.wire) {
+                    mcclx_seg g = z;
+                    g.out = r->tensors[q];
+                    g.in[0] = wire_of(0);
+                    g.count = r->numel;
+                    ph.dec_segs.push_back(g);
+                } else {
+                    ph.copies.push_back(mcclx_copy_desc{r->tensors[q], r->tensors[0], r->numel * ts});
+                }
+            }
+            return;
+        }
         mcclx_seg s = z;
         s.count = r->numel;
         if (bf16_only) {
@@ -436,8 +490,9 @@ int check_replay(mcclx_ctx* ctx, const mcclx_replay* r, bool* fused, bool* nothi
         if (!r->tensors[i]) return bad("replay: null tensor");
     Layout L = layout_of(r);
     if (L.total > 0 && (!r->workspace || r->workspace_bytes < L.total)) return bad("workspace too small");
-    // the binomial tree of more than MCCLX_MAX_INPUTS ranks does not cut into a chain of folds
-    *fused = r->mode == MCCLX_REPLAY_FUSED && (r->world <= MCCLX_MAX_INPUTS || r->algo != MCCLX_ALGO_TREE);
+    // the tree is fused as a tree of 8-rank trees: up to 8 x 8 ranks
+    *fused = r->mode == MCCLX_REPLAY_FUSED &&
+             (r->algo != MCCLX_ALGO_TREE || r->world <= MCCLX_MAX_INPUTS * MCCLX_MAX_INPUTS);
     return MCCLX_OK;
 }
 

@@ -79,13 +79,17 @@ def test_allreduce_other_ops_and_fp16(H, U, algo, op, mode):
 @pytest.mark.parametrize("algo", [RING, TREE, BUTTERFLY])
 def test_worlds_wider_than_one_fold(H, U, algo):
     """More ranks than one fold takes operands: ring and butterfly chain folds (8 operands, then
-    the partial result + 7 more, ...), the tree runs the stepwise schedule; all bit-exact."""
+    the partial result + 7 more, ...), the tree folds blocks of 8 ranks and then the blocks; all bit-exact."""
     run_case(H, U, algo, 11, F32, SUM, True, FUSED, 2003, seed=11)
     run_case(H, U, algo, 16, BF16, AVG, False, FUSED, 2003, seed=16)
     run_case(H, U, algo, 9, F32, AVG, False, FUSED, 40009, seed=9, specials=True)
     run_case(H, U, algo, 23, F32, AVG, True, FUSED, 5003, seed=23, specials=True)
     run_case(H, U, algo, 10, BF16, MAX, False, FUSED, 3001, seed=10)
     run_case(H, U, algo, 12, F32, PRODUCT, True, FUSED, 3001, seed=12)
+    if algo == TREE:     # a tree of 8-rank trees up to 64 ranks, the stepwise schedule beyond
+        for world, dtype, op, wire in ((17, F32, AVG, False), (33, F32, SUM, True), (64, BF16, SUM, False),
+                                       (57, F32, MIN, True), (65, F32, AVG, True)):
+            run_case(H, U, algo, world, dtype, op, wire, FUSED, 1237, seed=world)
 
 
 def test_tree_with_fewer_elements_than_ranks(H, U):  # ProcessGroupMCCL.cpp:143-145 -> tree
@@ -283,3 +287,5 @@ def test_launch_counts_of_the_fused_schedules(H, K, U):
     assert launches(lambda: H.allreduce_replay_many(groups, "sum", TREE)) == 2
     wide = [U.to_dev(U.rand_values(rng, n, F32), F32) for _ in range(16)]     # 16 ranks: folds of 8, 8 and 2 operands
     assert launches(lambda: H.allreduce_replay(wide, "avg", RING, wire_bf16=True, mode=FUSED)) == 1 + 3 + 1
+    small = [U.to_dev(U.rand_values(rng, 1000, F32), F32) for _ in range(20)]  # tree of 20: blocks 8 + 8 + 4, then 3
+    assert launches(lambda: H.allreduce_replay(small, "sum", TREE, mode=FUSED)) == 3 + 1
