@@ -654,10 +654,13 @@ int mcclx_reduce_scatter_replay(mcclx_ctx* ctx, int world, void* const* outs,
 int mcclx_allgather_replay(mcclx_ctx* ctx, int world, void* const* outs, const void* const* ins,
                            uint64_t chunk_nbytes) {
     if (!ctx || !outs || !ins || world < 1) return bad("allgather: bad argument");
+    std::vector<mcclx_copy_desc> copies;
+    copies.reserve((size_t)world * (size_t)world);
     for (int r = 0; r < world; ++r)
         for (int p = 0; p < world; ++p)  // ProcessGroupMCCL.cpp:256-270
-            TRY(mcclx_copy(ctx, at(outs[r], (uint64_t)p * chunk_nbytes), ins[p], chunk_nbytes));
-    return MCCLX_OK;
+            copies.push_back(mcclx_copy_desc{at(outs[r], (uint64_t)p * chunk_nbytes), ins[p], chunk_nbytes});
+    // small chunks go out in one launch, large ones stream one launch each
+    return mcclx_copy_batched(ctx, copies.data(), (uint32_t)copies.size());
 }
 
 }  // extern "C"
