@@ -42,7 +42,7 @@ namespace {
 #define MCCLX_TUNE_BLOCK 512
 #endif
 #ifndef MCCLX_TUNE_U
-#define MCCLX_TUNE_U 0  // 0: derive from the register budget of the plan
+#define MCCLX_TUNE_U 0  // 0: the measured best per plan (Cfg::U)
 #endif
 #ifndef MCCLX_TUNE_NT_LOAD
 #define MCCLX_TUNE_NT_LOAD 1
@@ -62,9 +62,6 @@ namespace {
 
 constexpr int kBlock = MCCLX_TUNE_BLOCK;  // wavefronts of 64 lanes
 
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-// Under-aligned views: element alignment is all the kernels may assume.
-
 // Every operand lives in global memory (HBM or host memory mapped into the
 // device).  Pointers that reach a kernel through a descriptor table are
 // generic to the compiler; these casts let it emit global_load/global_store
@@ -76,7 +73,9 @@ template <class T> __device__ __forceinline__ const MCCLX_GLOBAL T* gptr(const v
 template <class T> __device__ __forceinline__ MCCLX_GLOBAL T* gptr(void* p) {
     return (MCCLX_GLOBAL T*)p;
 }
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+// Under-aligned views: element alignment is all the kernels may assume.
 typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
 typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 typedef u32x2 u32x2_a2 __attribute__((aligned(2)));
@@ -153,11 +152,6 @@ struct Cfg {
         return W == MCCLX_F32 || (IO == MCCLX_IO_OWN_FIRST_F32 && k == 0) ||
                (IO == MCCLX_IO_OWN_LAST_F32 && k == K - 1);
     }
-    __host__ __device__ static constexpr int regs_per_pack() {
-        int r = 0;
-        for (int k = 0; k < K; ++k) r += (in_is_f32(k) || E == 8) ? 4 : 2;
-        return r;
-    }
     // Packets per lane per iteration.  Measured on MI355X (one block per tile,
     // no grid-stride looping): one packet per lane streams fastest for folds with
     // an fp32 stream; all-16-bit plans and the one-input codec passes (encode,
@@ -181,7 +175,7 @@ __device__ __forceinline__ RawPack load_raw(const void* p, uint64_t pack) {
     }
 }
 
-// Operand k of one packet as 8 floats holding W-representable values.
+// Operand k of one packet as E floats holding W-representable values.
 template <class C, int k>
 __device__ __forceinline__ void decode(const RawPack& r, float (&v)[C::E]) {
     if constexpr (C::in_is_f32(k)) {
@@ -420,8 +414,6 @@ __device__ __forceinline__ void fold_segment(const SegArgs& s, float scale, bool
 
 // ------------------------------------------------------------------ kernels
 
-// Up to kFewSegs segments passed by value in the kernel arguments: blockIdx.y
-// picks the segment, blockIdx.x strides over its packets.
 // Everything a block needs from the kernel arguments, fetched with ONE batch of
 // scalar loads and one wait.  Left to itself the compiler fetches the fields
 // where they are first used -- three dependent fetch-and-wait rounds before the
@@ -434,6 +426,8 @@ __device__ __forceinline__ void fetch_together(SegArgs& s, float& scale, int32_t
                    "+s"(has_scale), "+s"(grid));
 }
 
+// Up to kFewSegs segments passed by value in the kernel arguments: blockIdx.y
+// picks the segment, blockIdx.x strides over its packets.
 template <class C>
 __global__ void __launch_bounds__(kBlock) fold_few_kernel(FewArgs a) {
     SegArgs s = a.seg[blockIdx.y];
