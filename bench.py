@@ -284,6 +284,27 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
         for hptr in pin:
             q.host_free(hptr)
 
+    # the same fused fold over other bucket sizes (3 ranks, bf16 wire, x 1/3; cold: copies rotate
+    # over >= 600 MB): where the fixed cost of a launch stops mattering
+    sweep = {}
+    for mib in (1, 4, 16, 64, 256):
+        n = mib * (1 << 20) // 4
+        ncopies = max(2, min(256, (640 << 20) // (n * 12)))
+        ch = H.chunkize(n, 1, world)
+        bufs = [([torch.randn(n, device="cuda") * 1e-3 for _ in range(world)],
+                 [(torch.randn(n, device="cuda") * 1e-3).to(torch.bfloat16) for _ in range(world)]) for _ in range(ncopies)]
+
+        def sz_step(i, bufs=bufs, ch=ch, ncopies=ncopies):
+            ts, ws = bufs[i % ncopies]
+            q.fold(plan, [K.make_seg(ts[R].data_ptr() + 4 * st, 0,
+                                     [ts[R].data_ptr() + 4 * st] + [ws[p].data_ptr() + 2 * st for p in range(world) if p != R], c)
+                          for R, (st, c, _, _) in enumerate(ch)])
+        reps = max(10, min(200, (16 << 30) // (n * 12)))
+        ms, _ = measure(sz_step, reps, 5)
+        sweep[f"{mib}MiB"] = {"us": round(ms / reps * 1e3, 2), "GBps": round(gbs(n * 12, ms / reps), 1)}
+        del bufs
+    out["fold_by_bucket_size"] = sweep
+
     # encode leg: 3 ranks x (4 B read + 2 B write) per element
     def enc(i):
         s = i % sets
