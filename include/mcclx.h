@@ -170,6 +170,23 @@ MCCLX_API int mcclx_fold(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg
 MCCLX_API int mcclx_fold_batched(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs,
                        uint32_t nseg);
 
+/* The batched fold for callers that cannot allocate.  It has no counterpart
+ * in the reference: it exists for code under HIP graph capture, tight serving
+ * loops and harnesses that forbid hipMalloc.  Same arguments, checks and
+ * results as mcclx_fold_batched, but the call allocates nothing on the device
+ * or the host: up to 32 segments travel in the kernel
+ * arguments, more go through a descriptor table in a static device array
+ * (128 KiB per GPU, held until the process ends) that small writer kernels
+ * fill from their own arguments -- the whole call is kernel launches only.
+ * More than MCCLX_NOALLOC_MAX_SEGS segments are refused with MCCLX_ERR_INVALID.
+ * Every call on a GPU shares that GPU's array: calls on one context are
+ * ordered by its queue, calls that overlap on one GPU from different contexts
+ * race.  Nothing in the array needs to start at zero; each call overwrites the
+ * part it reads. */
+#define MCCLX_NOALLOC_MAX_SEGS 1024
+MCCLX_API int mcclx_fold_batched_noalloc(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs,
+                               uint32_t nseg);
+
 /* dst <- src, nbytes, on the reduce queue.  Replaces unstage_from_recv
  * (MPSInterop.mm:408-435) and the allgather legs (AllreduceAlgos.cpp:77-86,
  * ProcessGroupMCCL.cpp:232-273). */

@@ -14,6 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("MCCLX_LIBRARY") or os.path.join(HERE, "libmcclx.so")
 
 MAX_INPUTS = 8
+NOALLOC_MAX_SEGS = 1024
 
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_STATE, ERR_NOMEM = 0, -1, -2, -3, -4, -5
 F32, F16, BF16 = 0, 1, 2
@@ -74,6 +75,7 @@ SIGNATURES = {
     "mcclx_decode_bf16": (_i, [_vp, _vp, _vp, _u64]),
     "mcclx_fold": (_i, [_vp, C.POINTER(Plan), C.POINTER(Seg)]),
     "mcclx_fold_batched": (_i, [_vp, C.POINTER(Plan), C.POINTER(Seg), C.c_uint32]),
+    "mcclx_fold_batched_noalloc": (_i, [_vp, C.POINTER(Plan), C.POINTER(Seg), C.c_uint32]),
     "mcclx_copy": (_i, [_vp, _vp, _vp, _u64]),
     "mcclx_copy_batched": (_i, [_vp, C.POINTER(CopyDesc), C.c_uint32]),
     "mcclx_queue_drain": (_i, [_vp]),

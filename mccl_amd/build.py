@@ -19,7 +19,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(ROOT, "build", "mcclx")
 LIB_PATH = os.path.join(HERE, "libmcclx.so")
 
-SOURCES = ["fold_kernels.hip", "copy_kernel.hip", "mcclx_api.cpp", "mcclx_sched.cpp"]
+SOURCES = ["fold_kernels.hip", "copy_kernel.hip", "static_table.hip", "mcclx_api.cpp", "mcclx_sched.cpp"]
 FOLD_PARTS = 6  # fold_kernels.hip is compiled once per part (-DMCCLX_PART=n), in parallel
 HEADERS = ["fold_launch.h", "mcclx_internal.h", os.path.join(ROOT, "include", "mcclx.h")]
 

@@ -86,4 +86,18 @@ hipError_t launch_copy_many(hipStream_t st, const CopyTable& t, int align, uint3
 hipError_t launch_copy(hipStream_t st, void* dst, const void* src, uint64_t nbytes,
                        uint32_t max_blocks);
 
+// The allocation-free batched fold keeps its descriptor table in a static
+// device array of kStaticTableBytes (one per GPU): room for
+// MCCLX_NOALLOC_MAX_SEGS descriptors of 88 bytes plus their work-item prefix
+// sums.  `static_table_resolve` returns that array's address on `device`, which
+// must be the current device; `launch_table_write` stores up to kUploadWords
+// 8-byte words there, carried in the kernel arguments of a one-block launch.
+constexpr size_t kStaticTableBytes = 128 * 1024;
+constexpr uint32_t kUploadWords = 448;  // 3584 bytes of payload per writer launch
+static_assert((size_t)MCCLX_NOALLOC_MAX_SEGS * sizeof(SegArgs) +
+                  ((size_t)MCCLX_NOALLOC_MAX_SEGS + 1) * sizeof(uint64_t) <= kStaticTableBytes,
+              "the static table must hold the largest allocation-free launch");
+hipError_t static_table_resolve(int device, void** out);
+hipError_t launch_table_write(hipStream_t st, void* dst_words, const uint64_t* words, uint32_t n);
+
 }  // namespace mcclx

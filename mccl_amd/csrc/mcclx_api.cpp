@@ -98,6 +98,7 @@ struct mcclx_ctx {
     void* stage_recv[2] = {nullptr, nullptr};
     hipEvent_t stage_recv_done[2] = {nullptr, nullptr};
     bool stage_recv_pending[2] = {false, false};
+    void* static_table = nullptr;  // this device's copy of the static descriptor table (static_table.hip)
 };
 
 namespace {
@@ -357,6 +358,24 @@ int table_launched(mcclx_ctx* ctx, TableSlot* slot) {
     return MCCLX_OK;
 }
 
+// Descriptors in the kernel arguments (nseg <= kFewSegs).
+int launch_by_value(mcclx_ctx* ctx, const mcclx::PlanKey& key, float scale_f, int has_scale,
+                    const mcclx_seg* segs, uint32_t nseg) {
+    mcclx::LaunchParams lp;
+    lp.max_blocks = ctx->max_blocks;
+    mcclx::FewArgs a;
+    memset(&a, 0, sizeof a);
+    for (uint32_t s = 0; s < nseg; ++s) memcpy(&a.seg[s], &segs[s], sizeof(mcclx_seg));
+    a.scale = scale_f;
+    a.has_scale = has_scale;
+    a.nseg = (int32_t)nseg;
+    lp.few = &a;
+    hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
+    if (e != hipSuccess) return launch_error(e, key);
+    ++ctx->launches;
+    return MCCLX_OK;
+}
+
 int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uint32_t nseg) {
     if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
     mcclx::PlanKey key;
@@ -383,19 +402,7 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
         }
         by_value = longest * nseg <= 4 * total + 64;
     }
-    if (by_value) {
-        mcclx::FewArgs a;
-        memset(&a, 0, sizeof a);
-        for (uint32_t s = 0; s < nseg; ++s) memcpy(&a.seg[s], &segs[s], sizeof(mcclx_seg));
-        a.scale = scale_f;
-        a.has_scale = has_scale;
-        a.nseg = (int32_t)nseg;
-        lp.few = &a;
-        hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
-        if (e != hipSuccess) return launch_error(e, key);
-        ++ctx->launches;
-        return MCCLX_OK;
-    }
+    if (by_value) return launch_by_value(ctx, key, scale_f, has_scale, segs, nseg);
 
     // descriptor table: segs, then nseg+1 work-item prefix sums
     std::lock_guard<std::mutex> lk(ctx->mu);
@@ -476,6 +483,11 @@ int make_ctx(int device, hipStream_t borrowed, bool borrow, mcclx_ctx** out) {
         if (x >= 0 && x <= mcclx::kFewSegs) ctx->few_max = (uint32_t)x;
     }
     if (const char* v = getenv("MCCLX_VALIDATE")) ctx->validate = (v[0] == '1');
+    e = mcclx::static_table_resolve(device, &ctx->static_table);  // `device` is current (guard above)
+    if (e != hipSuccess) {
+        delete ctx;
+        return fail(MCCLX_ERR_HIP, "hipGetSymbolAddress(static table) failed: %s", hipGetErrorString(e));
+    }
     if (borrow) {
         ctx->stream = borrowed;
     } else {
@@ -550,6 +562,74 @@ int mcclx_fold(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* seg) {
 
 int mcclx_fold_batched(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uint32_t nseg) {
     return fold_impl(ctx, plan, segs, nseg);
+}
+
+int mcclx_fold_batched_noalloc(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uint32_t nseg) {
+    static_assert(sizeof(mcclx_seg) % 8 == 0, "descriptors are uploaded as 8-byte words");
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    if (nseg > MCCLX_NOALLOC_MAX_SEGS)
+        return fail(MCCLX_ERR_INVALID, "fold_batched_noalloc: %u segments, the static table holds at most %d",
+                    nseg, MCCLX_NOALLOC_MAX_SEGS);
+    mcclx::PlanKey key;
+    float scale_f;
+    int has_scale;
+    if (int rc = check_plan(plan, &key, &scale_f, &has_scale)) return rc;
+    if (int rc = check_segs(ctx, key, segs, nseg)) return rc;
+    if (nseg == 0) return MCCLX_OK;
+    DeviceGuard guard(ctx->device);
+    if (!guard.ok) return fail(MCCLX_ERR_HIP, "hipSetDevice(%d) failed", ctx->device);
+    if (nseg <= (uint32_t)mcclx::kFewSegs) return launch_by_value(ctx, key, scale_f, has_scale, segs, nseg);
+
+    uint64_t total = 0, uniform = mcclx::items_for(key, segs[0].count);
+    for (uint32_t s = 0; s < nseg; ++s) {
+        const uint64_t n = mcclx::items_for(key, segs[s].count);
+        if (n != uniform) uniform = 0;
+        total += n;
+    }
+    if (total == 0) return MCCLX_OK;
+    if (total >> 31) return fail(MCCLX_ERR_INVALID, "fold: more than 2^31 work items in one launch");
+
+    // Table layout, in 8-byte words: nseg descriptors, then nseg+1 work-item prefix
+    // sums.  It is produced a writer launch's worth at a time, on the stack.
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    constexpr uint32_t kSegWords = sizeof(mcclx_seg) / 8;
+    const uint32_t seg_words = nseg * kSegWords, words = seg_words + nseg + 1;
+    uint64_t* const table = static_cast<uint64_t*>(ctx->static_table);
+    uint64_t running = 0;  // work items of the segments before `next_prefix`
+    uint32_t next_prefix = 0;
+    for (uint32_t off = 0; off < words; off += mcclx::kUploadWords) {
+        uint64_t buf[mcclx::kUploadWords];
+        const uint32_t n = words - off < mcclx::kUploadWords ? words - off : mcclx::kUploadWords;
+        for (uint32_t i = 0; i < n; ++i) {
+            const uint32_t g = off + i;
+            if (g < seg_words) {
+                memcpy(&buf[i], reinterpret_cast<const char*>(segs) + (size_t)g * 8, 8);
+            } else {
+                buf[i] = running;
+                if (next_prefix < nseg) running += mcclx::items_for(key, segs[next_prefix].count);
+                ++next_prefix;
+            }
+        }
+        hipError_t e = mcclx::launch_table_write(ctx->stream, table + off, buf, n);
+        if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "table write launch failed: %s", hipGetErrorString(e));
+        ++ctx->launches;
+    }
+    mcclx::TableArgs t;
+    t.segs = reinterpret_cast<const mcclx::SegArgs*>(table);
+    t.first_item = table + seg_words;
+    t.item_map = nullptr;  // ragged segments: a block finds its segment by bisection over first_item
+    t.total_items = total;
+    t.uniform_items = uniform;
+    t.nseg = nseg;
+    t.scale = scale_f;
+    t.has_scale = has_scale;
+    mcclx::LaunchParams lp;
+    lp.max_blocks = ctx->max_blocks;
+    lp.table = &t;
+    hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
+    if (e != hipSuccess) return launch_error(e, key);
+    ++ctx->launches;
+    return MCCLX_OK;
 }
 
 int mcclx_reduce(mcclx_ctx* ctx, void* dst, const void* src, int dtype, uint64_t count, int op) {
