@@ -146,6 +146,15 @@ typedef struct {
     uint64_t count;  /* elements */
 } mcclx_seg;
 
+/* plan.flags.  By default every step of a fold computes op(dst = partial
+ * result, src = in[j]): the roles the butterfly, the tree and reduce_scatter
+ * give their operands (AllreduceAlgos.cpp:108-111,172-180,
+ * ProcessGroupMCCL.cpp:378-386).  The ring reduces the travelling partial
+ * result INTO the receiver's own chunk, op(dst = in[j], src = partial)
+ * (AllreduceAlgos.cpp:72-74); MIN and MAX keep dst on a tie or a NaN
+ * (shaders.metal:65-72), so they can tell the two apart. */
+#define MCCLX_PLAN_ACC_IS_SRC 1
+
 typedef struct {
     int32_t dtype;      /* W: MCCLX_F32 / F16 / BF16                                  */
     int32_t io;         /* MCCLX_IO_*  (non-PURE needs W = bf16)                      */
@@ -154,7 +163,7 @@ typedef struct {
     int32_t op;         /* MCCLX_SUM/AVG(=SUM)/PRODUCT/MIN/MAX                        */
     int32_t acc;        /* MCCLX_ACC_*                                                */
     int32_t scale_mode; /* MCCLX_SCALE_*; NONE ignores `scale`                        */
-    int32_t reserved;   /* must be 0                                                  */
+    int32_t flags;      /* MCCLX_PLAN_* bits, 0 otherwise                             */
     double scale;       /* e.g. 1.0 / world (AllreduceAlgos.cpp:88-91)                */
 } mcclx_plan;
 

@@ -25,6 +25,7 @@ TOPO_FOLD, TOPO_BINOMIAL = 0, 1
 ACC_STEP, ACC_F32 = 0, 1
 ALGO_RING, ALGO_TREE, ALGO_BUTTERFLY = 0, 1, 2
 REPLAY_STEPWISE, REPLAY_FUSED = 0, 1
+PLAN_ACC_IS_SRC = 1
 
 
 class Seg(C.Structure):
@@ -39,7 +40,7 @@ class CopyDesc(C.Structure):
 class Plan(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("io", C.c_int32), ("k", C.c_int32), ("topo", C.c_int32),
                 ("op", C.c_int32), ("acc", C.c_int32), ("scale_mode", C.c_int32),
-                ("reserved", C.c_int32), ("scale", C.c_double)]
+                ("flags", C.c_int32), ("scale", C.c_double)]
 
 
 class Chunk(C.Structure):

@@ -132,12 +132,17 @@ template <> struct Num<MCCLX_F16> {
 };
 
 // The reference's element operators.  min/max follow the Metal definition
-// "y if y < x else x" / "y if x < y else x" with x = accumulator (dst).
+// "y if y < x else x" / "y if x < y else x" with x = dst, y = src: dst is kept on
+// a tie (+0 against -0) and when either operand is NaN.  `a` is the accumulator,
+// `b` the next operand; by default the accumulator is dst, the *_ACC_SRC forms
+// (the ring's roles, AllreduceAlgos.cpp:72-74) make the next operand dst.
 template <int OP> __device__ __forceinline__ float apply(float a, float b) {
     if constexpr (OP == MCCLX_SUM) return a + b;
     else if constexpr (OP == MCCLX_PRODUCT) return a * b;
     else if constexpr (OP == MCCLX_MIN) return (b < a) ? b : a;
-    else return (a < b) ? b : a;
+    else if constexpr (OP == MCCLX_MAX) return (a < b) ? b : a;
+    else if constexpr (OP == MCCLX_MIN_ACC_SRC) return (a < b) ? a : b;
+    else return (b < a) ? a : b;  // MCCLX_MAX_ACC_SRC
 }
 
 // ------------------------------------------------------------ configuration
@@ -587,6 +592,8 @@ int plan_unroll(const PlanKey& key) {
         case MCCLX_PRODUCT: MCCLX_TOPO_CASES(W, MCCLX_IO_PURE, MCCLX_PRODUCT, MCCLX_ACC_STEP) \
         case MCCLX_MIN: MCCLX_TOPO_CASES(W, MCCLX_IO_PURE, MCCLX_MIN, MCCLX_ACC_STEP)   \
         case MCCLX_MAX: MCCLX_TOPO_CASES(W, MCCLX_IO_PURE, MCCLX_MAX, MCCLX_ACC_STEP)   \
+        case MCCLX_MIN_ACC_SRC: MCCLX_K_CASES(W, MCCLX_IO_PURE, MCCLX_TOPO_FOLD, MCCLX_MIN_ACC_SRC, MCCLX_ACC_STEP) \
+        case MCCLX_MAX_ACC_SRC: MCCLX_K_CASES(W, MCCLX_IO_PURE, MCCLX_TOPO_FOLD, MCCLX_MAX_ACC_SRC, MCCLX_ACC_STEP) \
         default: return hipErrorInvalidValue;                                           \
     }
 

@@ -44,6 +44,10 @@ struct TableArgs {
     int32_t has_scale;
 };
 
+// Kernel-side operator codes beyond the public MCCLX_* ones: MIN / MAX with the
+// accumulator in the reference's `src` role (plan flag MCCLX_PLAN_ACC_IS_SRC).
+enum { MCCLX_MIN_ACC_SRC = 5, MCCLX_MAX_ACC_SRC = 6 };
+
 struct PlanKey {
     int dtype, io, k, topo, op, acc;
 };

@@ -194,7 +194,7 @@ int normalize_op(int op, int* out) {
 
 int check_plan(const mcclx_plan* p, mcclx::PlanKey* key, float* scale_f, int* has_scale) {
     if (!p) return fail(MCCLX_ERR_INVALID, "plan is null");
-    if (p->reserved != 0) return fail(MCCLX_ERR_INVALID, "plan.reserved must be 0");
+    if (p->flags & ~MCCLX_PLAN_ACC_IS_SRC) return fail(MCCLX_ERR_INVALID, "plan.flags=%d has unknown bits", p->flags);
     if (!dtype_ok(p->dtype))
         return fail(MCCLX_ERR_UNSUPPORTED, "No kernel for dtype code %d", p->dtype);
     if (p->k < 1 || p->k > MCCLX_MAX_INPUTS)
@@ -216,6 +216,11 @@ int check_plan(const mcclx_plan* p, mcclx::PlanKey* key, float* scale_f, int* ha
         return fail(MCCLX_ERR_UNSUPPORTED, "fp16 folds round after every step (STEP) only");
     if (p->io == MCCLX_IO_OWN_LAST_F32 && p->topo == MCCLX_TOPO_BINOMIAL)
         return fail(MCCLX_ERR_UNSUPPORTED, "the tree reduces into rank 0: own operand is first");
+    if ((p->flags & MCCLX_PLAN_ACC_IS_SRC) && p->topo == MCCLX_TOPO_BINOMIAL && p->k >= 4)
+        return fail(MCCLX_ERR_UNSUPPORTED, "the tree reduces into the surviving rank: its partial result is dst");
+    // SUM and PRODUCT do not depend on the operand roles; MIN and MAX do
+    if ((p->flags & MCCLX_PLAN_ACC_IS_SRC) && (op == MCCLX_MIN || op == MCCLX_MAX))
+        op = (op == MCCLX_MIN) ? mcclx::MCCLX_MIN_ACC_SRC : mcclx::MCCLX_MAX_ACC_SRC;
     int acc = (p->dtype == MCCLX_F32) ? MCCLX_ACC_STEP : p->acc;  // fp32 has no rounding to skip
     *key = mcclx::PlanKey{p->dtype, p->io, p->k, (p->k >= 4) ? p->topo : MCCLX_TOPO_FOLD, op, acc};
     *has_scale = p->scale_mode != MCCLX_SCALE_NONE;

@@ -194,6 +194,9 @@ mcclx_plan base_plan(const mcclx_replay* r, const Layout& L, int k) {
     p.acc = r->acc;
     p.scale_mode = (r->op == MCCLX_AVG) ? MCCLX_SCALE_VIEW : MCCLX_SCALE_NONE;
     p.scale = 1.0 / (double)r->world;
+    // the ring reduces the travelling partial result into each receiver's own chunk:
+    // dst = the next operand, src = the partial result (AllreduceAlgos.cpp:72-74)
+    if (r->algo == MCCLX_ALGO_RING) p.flags = MCCLX_PLAN_ACC_IS_SRC;
     return p;
 }
 
@@ -287,6 +290,7 @@ void plan_phases(const mcclx_replay* r, const Layout& L, Phases& ph) {
     ph.enc = base_plan(r, L, 1);  // fp32 -> bf16 of what travels
     ph.enc.io = MCCLX_IO_OWN_FIRST_F32;
     ph.enc.op = MCCLX_SUM;
+    ph.enc.flags = 0;
     ph.enc.scale_mode = MCCLX_SCALE_NONE;
     ph.dec = ph.enc;              // bf16 -> fp32 on arrival
     ph.dec.io = MCCLX_IO_OUT_F32;

@@ -222,8 +222,8 @@ def make_seg(out=0, wire_out=0, inputs=(), count=0) -> L.Seg:
 
 
 def make_plan(dtype, k, io=L.IO_PURE, topo=L.TOPO_FOLD, op=L.SUM, acc=L.ACC_STEP,
-              scale_mode=L.SCALE_NONE, scale=0.0) -> L.Plan:
-    return L.Plan(dtype, io, k, topo, op, acc, scale_mode, 0, scale)
+              scale_mode=L.SCALE_NONE, scale=0.0, flags=0) -> L.Plan:
+    return L.Plan(dtype, io, k, topo, op, acc, scale_mode, flags, scale)
 
 
 # ---- tensor variants (MetalKernels.hpp:14-43) ------------------------------

@@ -76,6 +76,76 @@ def test_allreduce_other_ops_and_fp16(H, U, algo, op, mode):
     run_case(H, U, algo, 3, F16, AVG, False, mode, 5003, seed=2)
 
 
+def tie_and_nan_values(rng, n, dtype, world):
+    """Operands on which MIN / MAX depend on which side is dst: +0 against -0 (a tie
+    keeps dst) and NaN against numbers (a NaN on either side keeps dst), at positions
+    that differ from rank to rank, between ordinary values.  fp16 gets the zeros only
+    (the payload of an fp16 NaN is hardware-defined)."""
+    pool = np.array([0.0, -0.0, 1.0, -1.0, 0.0, -0.0] + ([] if dtype == F16 else [np.nan, -np.nan, np.nan]),
+                    dtype=np.float32)
+    out = []
+    for _ in range(world):
+        x = pool[rng.integers(0, pool.size, n)]
+        plain = rng.random(n) < 0.2
+        x[plain] = rng.standard_normal(int(plain.sum())).astype(np.float32)
+        if dtype == F32:
+            out.append(x)
+        elif dtype == BF16:
+            out.append(orc.encode_bf16(x))
+        else:
+            out.append(x.astype(np.float16).view(np.uint16))
+    return out
+
+
+@pytest.mark.parametrize("algo", [RING, TREE, BUTTERFLY])
+@pytest.mark.parametrize("op", [MIN, MAX])
+def test_min_max_operand_roles_on_ties_and_nans(H, U, algo, op):
+    """The reference's min/max keep dst on a +0/-0 tie and when an operand is NaN
+    (shaders.metal:65-72), and each schedule decides which operand is dst: the ring
+    reduces the travelling partial result into the receiver's own chunk
+    (AllreduceAlgos.cpp:72-74), the others reduce received data into the partial result.
+    FUSED == STEPWISE == oracle, bit for bit, for every schedule."""
+    rng = np.random.default_rng(500 + 10 * algo + op)
+    names = {RING: "ring", TREE: "tree", BUTTERFLY: "butterfly"}
+    for world in (2, 3, 4, 5, 9, 12):
+        for dtype, wire in ((F32, False), (BF16, False), (F16, False), (F32, True)):
+            xs = tie_and_nan_values(rng, 6007, dtype, world)
+            want = [x.copy() for x in xs]
+            rc = orc.allreduce(algo, want, dtype, op) if not wire else \
+                orc.pg_allreduce(want, dtype, op, wire_bf16=True, env_algo=names[algo])[0]
+            assert rc == 0
+            got = {}
+            for mode in (STEPWISE, FUSED):
+                d = [U.to_dev(x, dtype) for x in xs]
+                H.allreduce_replay(d, op, algo, wire_bf16=wire, mode=mode)
+                got[mode] = [U.bits(t) for t in d]
+                for r in range(world):
+                    w = U.np_bits(np.ascontiguousarray(want[r]))
+                    assert np.array_equal(got[mode][r], w), \
+                        f"{names[algo]} world={world} dtype={dtype} wire={wire} mode={mode} rank={r}: " \
+                        f"{int((got[mode][r] != w).sum())} elements differ from the oracle"
+            for r in range(world):
+                assert np.array_equal(got[STEPWISE][r], got[FUSED][r])
+
+
+@pytest.mark.parametrize("op", [MIN, MAX])
+def test_reduce_scatter_min_max_on_ties_and_nans(H, U, op):
+    rng = np.random.default_rng(600 + op)
+    CH = 3001
+    for world in (2, 3, 8, 11):
+        for dtype in (F32, BF16, F16):
+            ins = tie_and_nan_values(rng, CH * world, dtype, world)
+            want = [np.zeros(CH, dtype=ins[0].dtype) for _ in range(world)]
+            assert orc.reduce_scatter(want, ins, dtype, op) == 0
+            for mode in (STEPWISE, FUSED):
+                din = [U.to_dev(x, dtype) for x in ins]
+                dout = [torch.empty(CH, dtype=din[0].dtype, device="cuda") for _ in range(world)]
+                H.reduce_scatter_replay(dout, din, op, mode=mode)
+                for r in range(world):
+                    assert np.array_equal(U.bits(dout[r]), U.np_bits(np.ascontiguousarray(want[r]))), \
+                        (world, dtype, mode, r)
+
+
 @pytest.mark.parametrize("algo", [RING, TREE, BUTTERFLY])
 def test_worlds_wider_than_one_fold(H, U, algo):
     """More ranks than one fold takes operands: ring and butterfly chain folds (8 operands, then
