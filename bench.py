@@ -47,6 +47,9 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="headline only (used when profiling)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--timeline", action="store_true",
+                    help="instead of the JSON line, print where the time of one C2 launch goes: every block's "
+                         "start and end stamps from the instrumented build (python -m mccl_amd.build --timeline)")
     return ap.parse_args()
 
 
@@ -59,8 +62,14 @@ def main():
 
     import numpy as np
     import torch
-    from mccl_amd.build import ensure_built
+    from mccl_amd.build import ensure_built, TIMELINE_LIB_PATH
     ensure_built()
+    if args.timeline:
+        if not os.path.exists(TIMELINE_LIB_PATH):
+            print("bench.py --timeline needs the instrumented build: python -m mccl_amd.build --timeline",
+                  file=sys.stderr)
+            sys.exit(2)
+        os.environ["MCCLX_LIBRARY"] = TIMELINE_LIB_PATH
     from mccl_amd import _lib as L
     from mccl_amd import kernels as K
     from mccl_amd import harness as H
@@ -97,6 +106,11 @@ def main():
     q.drain()
 
     plan = K.make_plan(L.BF16, world, io=L.IO_OWN_FIRST_F32, op=L.SUM, scale_mode=L.SCALE_VIEW, scale=scale)
+
+    # Results go to buffers of their own, so that every step of every replay folds the
+    # seeded payload (folding in place would feed step n+8 the result of step n).  The
+    # in-place form the scheduler issues moves the same bytes; it is timed as an extra.
+    results = [[torch.empty_like(t) for t in ts] for ts in tensors]
 
     def step_segs(s, with_wire_out=False, out_tensors=None):
         segs = []
@@ -154,8 +168,11 @@ def main():
         q.graph_destroy(gk)
         return ms_dev, ms_wall
 
-    cold = lambda i: q.fold(plan, step_segs(i % args.sets))
-    warm = lambda i: q.fold(plan, step_segs(0))
+    cold = lambda i: q.fold(plan, step_segs(i % args.sets, out_tensors=results[i % args.sets]))
+    warm = lambda i: q.fold(plan, step_segs(0, out_tensors=results[0]))
+    if args.timeline:
+        timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure, bytes_per_step)
+        return
     cold_dev, cold_wall = measure(cold, args.steps, args.warmup)
     warm_dev, _ = measure(warm, args.steps, args.warmup)
 
@@ -223,9 +240,149 @@ def main():
             "value": round(bytes_per_step / b_all / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"the same C2 bucket (3 chunks, 78,643,200 algorithmic bytes) as reference-shaped passes "
                       f"(encode, 2 binary bf16 reduces, scale, decode); best of {reps_all} passes, OpenMP",
-            "single_thread_GBps": round(bytes_per_step / b_one / 1e9, 2), "host_cpus": os.cpu_count()}
+            "single_thread_GBps": round(bytes_per_step / b_one / 1e9, 2), "host_cpus": os.cpu_count(),
+            "cpu_model": cpu_model()}
     result["extra"] = extra
     print(json.dumps(result))
+
+
+def cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure, bytes_per_step):
+    """Where the time of one C2 launch goes.  The instrumented build stamps every block
+    (start, arguments fetched, last store issued; 100 MHz wall clock) into a device
+    buffer; 16 consecutive cold launches are recorded into one graph, replayed, and
+    their stamps reduced to: the launch-to-launch period, the span from the first block's
+    start to the last block's end, the gap between launches, and the ramp and drain
+    inside the span."""
+    import ctypes as C
+    lib = L.lib()
+    set_tl = lib.mcclx_tune_timeline
+    set_tl.restype, set_tl.argtypes = None, [C.c_void_p, C.c_uint64, C.c_uint64]
+    slots, per_slot, rec_words = 16, 4096, 4          # a record is 4 x 8 bytes
+    cus = q.compute_units
+    out = []
+    pr = out.append
+    pr("C2 fused fold -- timeline of one launch from per-block time stamps, MI355X (gfx950)")
+    pr("")
+    pr("Command: python -m mccl_amd.build --timeline   (here, once)   then on the GPU box:   python bench.py --timeline")
+    pr("Every block of fold_few_kernel<bf16, own-first fp32, k=3> records wall_clock64() (100 MHz, 10 ns ticks) at its first")
+    pr("instruction, once its kernel arguments have arrived, and after its last store was issued. 16 consecutive launches")
+    pr("(3201 blocks of 512 threads each: one per 8 KiB tile of a chunk; cold = rotating 8 copies of the workload,")
+    pr("944 MB + 629 MB of results) are recorded into one HIP graph; figures are means over launches 3..15 of its 4th replay.")
+    pr("All times in microseconds.")
+
+    def capture(seg_fn, label):
+        buf = torch.zeros(slots * per_slot * rec_words, dtype=torch.int64, device="cuda")
+        torch.cuda.synchronize()
+        set_tl(buf.data_ptr(), slots, per_slot)
+        q.graph_begin()
+        for i in range(slots):
+            seg_fn(i)
+        g = q.graph_end()
+        set_tl(None, 0, 0)
+        for _ in range(4):
+            q.graph_launch(g)
+            q.drain()
+        q.graph_destroy(g)
+        rec = buf.cpu().numpy().reshape(slots, per_slot, rec_words)
+        launches = []
+        for i in range(slots):
+            r = rec[i]
+            r = r[r[:, 2] != 0]
+            t0, ta, t1 = r[:, 0].astype(np.int64), r[:, 1].astype(np.int64), r[:, 2].astype(np.int64)
+            xcc = ((r[:, 3].view(np.uint64) >> np.uint64(32)) & np.uint64(15)).astype(np.int64)
+            launches.append((t0, ta, t1, xcc))
+        tick = 0.01
+        rows = []
+        for i in range(2, slots - 1):
+            t0, ta, t1, xcc = launches[i]
+            n0 = launches[i + 1][0]
+            s0, e1 = t0.min(), t1.max()
+            st = np.sort(t0)
+            en = np.sort(t1)
+            fill_n = min(len(st), 4 * cus) - 1
+            per_x = [t1[xcc == x].max() - s0 for x in range(8) if (xcc == x).any()]
+            rows.append(dict(
+                blocks=len(t0), period=(n0.min() - s0) * tick, span=(e1 - s0) * tick, gap=(n0.min() - e1) * tick,
+                fill=(st[fill_n] - s0) * tick, args=float((ta - t0).mean()) * tick, first_end=(en[0] - s0) * tick,
+                life=float((t1 - t0).mean()) * tick, last_start=(st[-1] - s0) * tick,
+                last90=(e1 - en[int(0.9 * len(en))]) * tick, xcd_spread=(max(per_x) - min(per_x)) * tick))
+        m = {k: float(np.mean([r[k] for r in rows])) for k in rows[0]}
+        pr("")
+        pr(f"[{label}]")
+        pr(f"  blocks per launch                                   {int(m['blocks'])}")
+        pr(f"  period: first block start -> next launch's first    {m['period']:6.2f}   = {bytes_per_step / m['period'] / 1e3:6.0f} GB/s algorithmic")
+        pr(f"  span:   first block start -> last block's end       {m['span']:6.2f}")
+        pr(f"  gap:    last block's end -> next launch's first     {m['gap']:6.2f}   (store acknowledgements, end-of-kernel release, dispatch of the next)")
+        pr(f"  inside the span:")
+        pr(f"    {4 * cus} blocks (all wave slots) started after        {m['fill']:6.2f}")
+        pr(f"    a block waits for its kernel arguments            {m['args']:6.2f}   (mean)")
+        pr(f"    first block has its data and ends after           {m['first_end']:6.2f}   (nothing has been written before this)")
+        pr(f"    mean block lifetime, start -> last store issued   {m['life']:6.2f}")
+        pr(f"    last block starts at                              {m['last_start']:6.2f}")
+        pr(f"    the last 10 % of block ends take                  {m['last90']:6.2f}   (a tenth of the span would be {0.1 * m['span']:.2f})")
+        pr(f"    spread of the 8 XCDs' finishing times             {m['xcd_spread']:6.2f}")
+        # one launch in 1 us bins
+        t0, ta, t1, xcc = launches[8]
+        s0 = t0.min()
+        pr(f"  launch 9 of the 16, per microsecond since its first block started:")
+        pr(f"    t       started   ended   resident   GB/s by block ends")
+        per_block = bytes_per_step / len(t0)
+        for b in range(0, int((t1.max() - s0) * tick) + 1):
+            lo, hi = s0 + b * 100, s0 + (b + 1) * 100
+            st_n = int(((t0 >= lo) & (t0 < hi)).sum())
+            en_n = int(((t1 >= lo) & (t1 < hi)).sum())
+            res = int(((t0 < hi) & (t1 >= hi)).sum())
+            pr(f"    {b:2d}-{b + 1:<2d}   {st_n:6d}  {en_n:6d}   {res:6d}     {en_n * per_block / 1e-6 / 1e9:7.0f}")
+        return m
+
+    sets = args.sets
+    cold = capture(lambda i: q.fold(plan, step_segs(i % sets, out_tensors=results[i % sets])), "cold: rotating copies, reads from HBM")
+    warm = capture(lambda i: q.fold(plan, step_segs(0, out_tensors=results[0])), "warm: one copy, resident in the 256 MiB Infinity Cache")
+
+    # the same launch without the stamps, and what bounds it: one-directional streams of the same footprint
+    gbs = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
+    steps = args.steps
+    ms, _ = measure(lambda i: q.fold(plan, step_segs(i % sets, out_tensors=results[i % sets])), steps, args.warmup)
+    fold_us = ms / steps * 1e3
+    fp = bytes_per_step
+    probe = torch.randint(0, 256, (8 * fp,), dtype=torch.uint8, device="cuda")
+    lines = []
+    for nbytes, write, name in ((fp, False, "read only,  78,643,200 B"), (fp, True, "write only, 78,643,200 B"),
+                                (fp * 2 // 3, False, "read only,  52,428,800 B (the fold's reads)"),
+                                (fp // 3, True, "write only, 26,214,400 B (the fold's writes)")):
+        ms, _ = measure(lambda i, nbytes=nbytes, write=write: q.probe_stream(probe.data_ptr() + (i % 8) * fp, nbytes, write),
+                        steps, args.warmup)
+        lines.append((name, ms / steps * 1e3, gbs(nbytes, ms / steps)))
+    ms, _ = measure(lambda i: q.copy(probe.data_ptr() + (i % 8) * fp, probe.data_ptr() + (i % 8) * fp + fp // 2, fp // 2),
+                    steps, args.warmup)
+    lines.append(("plain copy, 39,321,600 B in + 39,321,600 B out", ms / steps * 1e3, gbs(fp, ms / steps)))
+    ms, _ = measure(lambda i: q.probe_stream(probe.data_ptr(), 16 * 256, False), steps, args.warmup)
+    empty_us = ms / steps * 1e3
+    pr("")
+    pr(f"[the same launches without stamps, {steps} per graph replay, HIP events around the replay; cold]")
+    pr(f"  C2 fold (52.4 MB read + 26.2 MB written)            {fold_us:6.2f} us per launch = {gbs(fp, fold_us * 1e-3):6.0f} GB/s = {gbs(fp, fold_us * 1e-3) / 80:5.1f} % of 8 TB/s")
+    for name, us, g in lines:
+        pr(f"  {name:<50s}  {us:6.2f} us per launch = {g:6.0f} GB/s")
+    pr(f"  one-block launch (4 KiB read), back to back         {empty_us:6.2f} us per launch: what two dependent launches cost with no work in them")
+    pr("")
+    pr("Reading: a launch's period = gap + span. The gap (last store issued -> first block of the next launch running) is")
+    pr("spent on store acknowledgements, the end-of-kernel cache release and the dispatch of the dependent launch; the span")
+    pr("opens with one memory latency in which no byte has arrived and closes with a drain in which the queues empty.")
+    pr(f"Cold: {cold['gap']:.2f} gap + {cold['first_end']:.2f} until the first block has data leave "
+       f"{cold['period'] - cold['gap'] - cold['first_end']:.2f} us in which {fp / 1e6:.1f} MB move: "
+       f"{fp / (cold['period'] - cold['gap'] - cold['first_end']) / 1e3:.0f} GB/s while data flows.")
+    print("\n".join(out))
 
 
 def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_segs, measure, gbs):
@@ -249,6 +406,21 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
                     10, 2)
     out["plain_copy_1GiB_GBps"] = round(gbs(2 << 30, ms / 10), 1)
     del big
+
+    # one-directional ceilings at the bucket launch's own footprint (78,643,200 B, cold-rotated): a
+    # launch that only reads that many bytes and one that only writes them
+    fp = numel * 12
+    probe = torch.randint(0, 256, (8 * fp,), dtype=torch.uint8, device="cuda")
+    for write, name in ((False, "read_only"), (True, "write_only")):
+        ms, _ = measure(lambda i, write=write: q.probe_stream(probe.data_ptr() + (i % 8) * fp, fp, write), steps, warm)
+        out[f"{name}_same_footprint_us"] = round(ms / steps * 1e3, 2)
+        out[f"{name}_same_footprint_GBps"] = round(gbs(fp, ms / steps), 1)
+    del probe
+
+    # the fold as the scheduler issues it: result written in place over the owner's fp32 chunk
+    ms, _ = measure(lambda i: q.fold(plan, step_segs(i % sets)), steps, warm)
+    out["c2_fold_in_place_us"] = round(ms / steps * 1e3, 2)
+    out["c2_fold_in_place_GBps"] = round(gbs(numel * 12, ms / steps), 1)
 
     # C2 with the bf16 wire copy for the allgather leg also written (14 B/elem)
     ms, _ = measure(lambda i: q.fold(plan, step_segs(i % sets, with_wire_out=True)), steps, warm)

@@ -235,6 +235,12 @@ MCCLX_API int mcclx_event_wait(mcclx_ctx* ctx, uint64_t ticket);
 MCCLX_API int mcclx_timer_begin(mcclx_ctx* ctx);
 MCCLX_API int mcclx_timer_end(mcclx_ctx* ctx, float* elapsed_ms);
 
+/* Measurement aid: one launch that only reads (write = 0) or only writes
+ * (write = 1) nbytes of `buf` (4-byte aligned; its contents are unspecified
+ * afterwards) with the copy kernel's access shape -- the one-directional
+ * ceilings a fold launch of the same footprint is compared with. */
+MCCLX_API int mcclx_probe_stream(mcclx_ctx* ctx, void* buf, uint64_t nbytes, int write);
+
 /* ---- launch graphs ---------------------------------------------------------- */
 
 /* Gradient buckets have fixed shapes and addresses, so the launches of one

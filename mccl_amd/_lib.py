@@ -10,8 +10,9 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-# MCCLX_LIBRARY names a differently built libmcclx.so (tuning builds); default: the in-tree one.
-LIB_PATH = os.environ.get("MCCLX_LIBRARY") or os.path.join(HERE, "libmcclx.so")
+# The in-tree library.  MCCLX_LIBRARY, read when the library is first loaded, names a
+# differently built libmcclx.so (tuning builds).
+LIB_PATH = os.path.join(HERE, "libmcclx.so")
 
 MAX_INPUTS = 8
 NOALLOC_MAX_SEGS = 1024
@@ -79,6 +80,7 @@ SIGNATURES = {
     "mcclx_fold_batched_noalloc": (_i, [_vp, C.POINTER(Plan), C.POINTER(Seg), C.c_uint32]),
     "mcclx_copy": (_i, [_vp, _vp, _vp, _u64]),
     "mcclx_copy_batched": (_i, [_vp, C.POINTER(CopyDesc), C.c_uint32]),
+    "mcclx_probe_stream": (_i, [_vp, _vp, _u64, _i]),
     "mcclx_queue_drain": (_i, [_vp]),
     "mcclx_queue_wait_stream": (_i, [_vp, _vp]),
     "mcclx_stream_wait_queue": (_i, [_vp, _vp]),
@@ -128,11 +130,12 @@ def lib() -> C.CDLL:
         # first: then libmcclx binds to the runtime that owns torch's tensors.  The
         # other order loads both runtimes and corrupts the heap at exit.
         import torch  # noqa: F401
-        if not os.path.exists(LIB_PATH):
+        path = os.environ.get("MCCLX_LIBRARY") or LIB_PATH
+        if not os.path.exists(path):
             raise MCCLError(
-                f"[MCCL] native library {LIB_PATH} is missing: build it with "
+                f"[MCCL] native library {path} is missing: build it with "
                 "`python -m mccl_amd.build` (there is no fallback path)")
-        L = C.CDLL(LIB_PATH)
+        L = C.CDLL(path)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(L, name)  # AttributeError if the symbol is not exported
             fn.restype = res

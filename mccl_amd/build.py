@@ -147,6 +147,26 @@ def build_backend(verbose: bool = False) -> str:
     return out_path
 
 
+TIMELINE_LIB_PATH = os.path.join(HERE, "libmcclx_timeline.so")
+
+
+def build_timeline(verbose: bool = False) -> str:
+    """The tuning build bench.py --timeline loads: the same sources with
+    -DMCCLX_TUNE_TIMELINE=1 (every block of a by-value fold launch records its start
+    and end times) and only the measured plans instantiated, in one translation unit
+    per source.  Written to mccl_amd/libmcclx_timeline.so; the shipped library is
+    not touched."""
+    cc = hipcc()
+    cmd = [cc] + HIPCC_FLAGS + ["-DMCCLX_TUNE_TIMELINE=1", "-DMCCLX_TUNE_MINIMAL=1", "-x", "hip", "-shared",
+                                "-o", TIMELINE_LIB_PATH] + [os.path.join(CSRC, s) for s in SOURCES]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on the timeline build:\n{r.stdout}")
+    return TIMELINE_LIB_PATH
+
+
 def ensure_built() -> None:
     """Load what is built; build only if nothing is (used by bench.py and the smoke check)."""
     if not os.path.exists(LIB_PATH):
@@ -157,3 +177,5 @@ if __name__ == "__main__":
     print(build(force="--force" in sys.argv or needs_build(), verbose=True))
     if "--backend" in sys.argv:
         print(build_backend(verbose=True))
+    if "--timeline" in sys.argv:
+        print(build_timeline(verbose=True))

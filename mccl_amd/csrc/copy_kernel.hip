@@ -61,6 +61,27 @@ __global__ void __launch_bounds__(kBlock) copy_kernel(uint8_t* dst, const uint8_
         if (i < nbytes) gd[i] = gs[i];
     }
 }
+// One-directional streams with the copy kernel's access shape: what a launch
+// that only reads, or only writes, nbytes costs.  The read keeps its loads alive
+// through a store no input takes (packet XOR == magic, into the buffer's first
+// word).
+template <bool WRITE>
+__global__ void __launch_bounds__(kBlock) stream_probe_kernel(uint8_t* buf, uint64_t nbytes, uint32_t magic) {
+    typedef typename Packet<4>::type V;
+    MCCLX_GLOBAL uint8_t* g = (MCCLX_GLOBAL uint8_t*)buf;
+    const uint64_t P = nbytes / 16;
+    const uint64_t p = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (p >= P) return;
+    if (WRITE) {
+        const uint32_t w = (uint32_t)p * 2654435761u;
+        COPY_ST((MCCLX_GLOBAL V*)(g + p * 16), (u32x4{w, w ^ magic, ~w, w + magic}));
+    } else {
+        u32x4 v = COPY_LD((const MCCLX_GLOBAL V*)(g + p * 16));
+        const uint32_t x = v[0] ^ v[1] ^ v[2] ^ v[3];
+        if (x == magic) *(MCCLX_GLOBAL uint32_t*)g = x;
+    }
+}
+
 __device__ __forceinline__ uint32_t uni32(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
 __device__ __forceinline__ uint64_t uni64(uint64_t v) {
     return ((uint64_t)uni32((uint32_t)(v >> 32)) << 32) | uni32((uint32_t)v);
@@ -138,6 +159,18 @@ hipError_t launch_copy_many(hipStream_t st, const CopyTable& t, int align, uint3
         copy_many_kernel<2><<<dim3(g), dim3(kBlock), 0, st>>>(t);
     else
         copy_many_kernel<1><<<dim3(g), dim3(kBlock), 0, st>>>(t);
+    return hipGetLastError();
+}
+
+hipError_t launch_stream_probe(hipStream_t st, void* buf, uint64_t nbytes, bool write) {
+    const uint64_t g = (nbytes / 16 + kBlock - 1) / kBlock;
+    if (g == 0) return hipSuccess;
+    if (g >> 31) return hipErrorInvalidValue;
+    uint8_t* b = static_cast<uint8_t*>(buf);
+    if (write)
+        stream_probe_kernel<true><<<dim3((uint32_t)g), dim3(kBlock), 0, st>>>(b, nbytes, 0x9E3779B9u);
+    else
+        stream_probe_kernel<false><<<dim3((uint32_t)g), dim3(kBlock), 0, st>>>(b, nbytes, 0x9E3779B9u);
     return hipGetLastError();
 }
 

@@ -423,23 +423,37 @@ __device__ __forceinline__ void fold_segment(const SegArgs& s, float scale, bool
 // scalar loads and one wait.  Left to itself the compiler fetches the fields
 // where they are first used -- three dependent fetch-and-wait rounds before the
 // block can issue its first data load, 0.2-0.3 us per block on a kernel whose
-// blocks live for 4 us.  The empty asm makes every field live at one point.
+// blocks live for 2 us.  The empty asm makes every field live at one point.
+// Only the K operand pointers the plan reads are fetched: scalar registers are
+// what decides how many blocks a CU holds (see fold_few_kernel).
+template <int K>
 __device__ __forceinline__ void fetch_together(SegArgs& s, float& scale, int32_t& has_scale, uint32_t& grid) {
-    asm volatile(""
-                 : "+s"(s.out), "+s"(s.wire_out), "+s"(s.in[0]), "+s"(s.in[1]), "+s"(s.in[2]), "+s"(s.in[3]),
-                   "+s"(s.in[4]), "+s"(s.in[5]), "+s"(s.in[6]), "+s"(s.in[7]), "+s"(s.count), "+s"(scale),
-                   "+s"(has_scale), "+s"(grid));
+    asm volatile("" : "+s"(s.out), "+s"(s.wire_out), "+s"(s.count), "+s"(scale), "+s"(has_scale), "+s"(grid));
+#pragma unroll
+    for (int k = 0; k < K; ++k) asm volatile("" : "+s"(s.in[k]));
 }
 
 // Up to kFewSegs segments passed by value in the kernel arguments: blockIdx.y
 // picks the segment, blockIdx.x strides over its packets.
+//
+// Occupancy: a CU holds four 512-thread blocks (8 waves per SIMD) only while a
+// wave's scalar registers fit an allocation of 80 -- measured on MI355X: a
+// kernel with more starts 768 blocks at launch instead of 1024 and streams
+// 2-4 % slower.  Six registers are set aside on top of what the code uses (VCC,
+// flat scratch, XNACK mask), so the code itself has 74.
 template <class C>
-__global__ void __launch_bounds__(kBlock) fold_few_kernel(FewArgs a) {
+__device__ __forceinline__ void fold_few_body(const FewArgs& a) {
+#if MCCLX_TUNE_TIMELINE
+    const uint64_t t_start = wall_clock64();
+#endif
     SegArgs s = a.seg[blockIdx.y];
     float scale = a.scale;
     int32_t has_scale = a.has_scale;
     uint32_t grid = gridDim.x;
-    fetch_together(s, scale, has_scale, grid);
+    fetch_together<C::K>(s, scale, has_scale, grid);
+#if MCCLX_TUNE_TIMELINE
+    const uint64_t t_args = wall_clock64();
+#endif
     const uint64_t span = (uint64_t)C::U * kBlock;
 #if MCCLX_TUNE_XCD
     // workgroups go to the XCDs round robin: block b runs on XCD b % N
@@ -450,7 +464,29 @@ __global__ void __launch_bounds__(kBlock) fold_few_kernel(FewArgs a) {
     fold_segment<C>(s, scale, has_scale != 0, (uint64_t)blockIdx.x * span, (uint64_t)grid * span,
                     blockIdx.x == 0);
 #endif
+#if MCCLX_TUNE_TIMELINE
+    if (a.timeline && threadIdx.x == 0) {
+        TimelineRecord r;
+        r.t_start = t_start;
+        r.t_args = t_args;
+        r.t_end = wall_clock64();
+        r.hw_id = __builtin_amdgcn_s_getreg((31 << 11) | 4);    // HW_ID: wave, SIMD, CU, SH, SE
+        r.xcc_id = __builtin_amdgcn_s_getreg((31 << 11) | 20);  // XCC_ID
+        a.timeline[(uint64_t)blockIdx.y * gridDim.x + blockIdx.x] = r;
+    }
+#endif
 }
+
+// Plans whose vector registers allow 8 waves per SIMD are held to 74 scalar
+// registers (a handful of spills into vector-register lanes); wide folds, which
+// the vector registers already limit to fewer waves, keep what they need.
+#define MCCLX_SGPR_CAP __attribute__((amdgpu_num_sgpr(80)))
+template <class C> constexpr bool kLightPlan = C::K <= 4;
+
+template <class C>
+__global__ void __launch_bounds__(kBlock) MCCLX_SGPR_CAP fold_few_kernel(FewArgs a) { fold_few_body<C>(a); }
+template <class C>
+__global__ void __launch_bounds__(kBlock) fold_few_wide_kernel(FewArgs a) { fold_few_body<C>(a); }
 
 // A value that is the same in every lane, moved to scalar registers.  The
 // compiler cannot always prove it (a quotient comes out of the vector ALU), and
@@ -471,7 +507,7 @@ __device__ __forceinline__ P* uniptr(P* p) {
 // The loop bound is fixed at launch, so every wave exits.  total_items < 2^31
 // (checked by the host).
 template <class C>
-__global__ void __launch_bounds__(kBlock) fold_table_kernel(TableArgs a) {
+__device__ __forceinline__ void fold_table_body(const TableArgs& a) {
     const uint64_t span = (uint64_t)C::U * kBlock;
     const uint32_t total = (uint32_t)a.total_items;
     const uint32_t uniform = (uint32_t)a.uniform_items;
@@ -508,7 +544,29 @@ __global__ void __launch_bounds__(kBlock) fold_table_kernel(TableArgs a) {
     }
 }
 
+template <class C>
+__global__ void __launch_bounds__(kBlock) MCCLX_SGPR_CAP fold_table_kernel(TableArgs a) { fold_table_body<C>(a); }
+template <class C>
+__global__ void __launch_bounds__(kBlock) fold_table_wide_kernel(TableArgs a) { fold_table_body<C>(a); }
+
 // ----------------------------------------------------------------- dispatch
+
+#if MCCLX_TUNE_TIMELINE
+// Where the next by-value launches put their records: a caller-provided device
+// buffer cut into `slots` regions of `per_slot` records, used round robin.
+static TimelineRecord* g_tl_buf = nullptr;
+static uint64_t g_tl_slots = 0, g_tl_per_slot = 0, g_tl_next = 0;
+static TimelineRecord* timeline_next(uint64_t blocks) {
+    if (!g_tl_buf || blocks > g_tl_per_slot) return nullptr;
+    return g_tl_buf + (g_tl_next++ % g_tl_slots) * g_tl_per_slot;
+}
+extern "C" MCCLX_API void mcclx_tune_timeline(void* device_buf, uint64_t slots, uint64_t records_per_slot) {
+    g_tl_buf = static_cast<TimelineRecord*>(device_buf);
+    g_tl_slots = slots;
+    g_tl_per_slot = records_per_slot;
+    g_tl_next = 0;
+}
+#endif
 
 template <class C>
 static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
@@ -517,7 +575,10 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
         TableArgs a = *lp.table;
         uint32_t grid = (uint32_t)(a.total_items < lp.max_blocks ? a.total_items : lp.max_blocks);
         if (grid == 0) return hipSuccess;
-        fold_table_kernel<C><<<dim3(grid), dim3(kBlock), 0, st>>>(a);
+        if constexpr (kLightPlan<C>)
+            fold_table_kernel<C><<<dim3(grid), dim3(kBlock), 0, st>>>(a);
+        else
+            fold_table_wide_kernel<C><<<dim3(grid), dim3(kBlock), 0, st>>>(a);
     } else {
         FewArgs a = *lp.few;
         uint64_t maxc = 0;
@@ -530,7 +591,13 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
 #if MCCLX_TUNE_XCD
         gx = (gx + MCCLX_TUNE_XCD - 1) / MCCLX_TUNE_XCD * MCCLX_TUNE_XCD;
 #endif
-        fold_few_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(kBlock), 0, st>>>(a);
+#if MCCLX_TUNE_TIMELINE
+        a.timeline = timeline_next(gx * (uint64_t)a.nseg);
+#endif
+        if constexpr (kLightPlan<C>)
+            fold_few_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(kBlock), 0, st>>>(a);
+        else
+            fold_few_wide_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(kBlock), 0, st>>>(a);
     }
     return hipGetLastError();
 }

@@ -26,11 +26,25 @@ struct SegArgs {
 };
 static_assert(sizeof(SegArgs) == sizeof(mcclx_seg), "SegArgs must mirror mcclx_seg");
 
+// Launch-timeline instrumentation (a tuning build only, -DMCCLX_TUNE_TIMELINE=1):
+// every block of a by-value fold launch records when it started, when its
+// arguments had arrived and when it had issued its last store.
+#ifndef MCCLX_TUNE_TIMELINE
+#define MCCLX_TUNE_TIMELINE 0
+#endif
+struct TimelineRecord {
+    uint64_t t_start, t_args, t_end;  // 100 MHz wall clock (10 ns ticks)
+    uint32_t hw_id, xcc_id;           // where the block ran: HW_ID register, XCC_ID register
+};
+
 struct FewArgs {
     SegArgs seg[kFewSegs];
     float scale;        // the constant as the fp32 value the kernel multiplies by
     int32_t has_scale;
     int32_t nseg;
+#if MCCLX_TUNE_TIMELINE
+    TimelineRecord* timeline;  // this launch's records, one per block (x fastest, then y), or null
+#endif
 };
 
 struct TableArgs {
@@ -89,6 +103,10 @@ hipError_t launch_copy_many(hipStream_t st, const CopyTable& t, int align, uint3
 // the memory counters): dst <- src, nbytes.
 hipError_t launch_copy(hipStream_t st, void* dst, const void* src, uint64_t nbytes,
                        uint32_t max_blocks);
+
+// Reads (write == false) or writes nbytes of `buf` once, one 16-byte packet per
+// lane like the copy kernel: the one-directional ceilings of a launch of that size.
+hipError_t launch_stream_probe(hipStream_t st, void* buf, uint64_t nbytes, bool write);
 
 // The allocation-free batched fold keeps its descriptor table in a static
 // device array of kStaticTableBytes (one per GPU): room for

@@ -710,6 +710,19 @@ int mcclx_copy(mcclx_ctx* ctx, void* dst, const void* src, uint64_t nbytes) {
     return MCCLX_OK;
 }
 
+int mcclx_probe_stream(mcclx_ctx* ctx, void* buf, uint64_t nbytes, int write) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    if (nbytes == 0) return MCCLX_OK;
+    if (!buf || (uintptr_t)buf % 4) return fail(MCCLX_ERR_INVALID, "probe_stream: buffer is null or not 4-byte aligned");
+    if (ctx->validate)
+        if (int rc = check_range(buf, nbytes, "buf", 0)) return rc;
+    DeviceGuard guard(ctx->device);
+    hipError_t e = mcclx::launch_stream_probe(ctx->stream, buf, nbytes, write != 0);
+    if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "probe launch failed: %s", hipGetErrorString(e));
+    ++ctx->launches;
+    return MCCLX_OK;
+}
+
 int mcclx_copy_batched(mcclx_ctx* ctx, const mcclx_copy_desc* descs, uint32_t n) {
     if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
     if (n == 0) return MCCLX_OK;

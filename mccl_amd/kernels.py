@@ -185,6 +185,10 @@ class ReduceQueue:
     def copy(self, dst_ptr: int, src_ptr: int, nbytes: int) -> None:
         L.check(L.lib().mcclx_copy(self.handle, C.c_void_p(dst_ptr), C.c_void_p(src_ptr), nbytes))
 
+    def probe_stream(self, ptr: int, nbytes: int, write: bool) -> None:
+        """One read-only or write-only pass over a buffer (measurement aid)."""
+        L.check(L.lib().mcclx_probe_stream(self.handle, C.c_void_p(ptr), nbytes, int(write)))
+
     def copy_batched(self, triples) -> None:
         """Many (dst, src, nbytes) copies in one launch (a few large ones go out one by one)."""
         arr = (L.CopyDesc * len(triples))(*[L.CopyDesc(d, s, n) for d, s, n in triples])
