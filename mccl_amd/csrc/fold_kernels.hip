@@ -31,6 +31,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "fold_launch.h"
 
@@ -169,7 +170,7 @@ struct Cfg {
 typedef u32x4 RawPack;  // one packet of one operand: 16 B, or 8 B in .xy (16-bit operand, E = 4)
 
 template <class C, int k>
-__device__ __forceinline__ RawPack load_raw(const void* p, uint64_t pack) {
+__device__ __forceinline__ RawPack load_raw(const void* p, uint32_t pack) {
     if constexpr (C::in_is_f32(k)) {
         return MCCLX_LDG(gptr<u32x4_a4>(static_cast<const float*>(p) + pack * C::E));
     } else if constexpr (C::E == 8) {
@@ -213,7 +214,7 @@ __device__ __forceinline__ float finish(float acc, float scale, bool has_scale) 
 }
 
 template <class C, int k, int U>
-__device__ __forceinline__ void load_all(const SegArgs& s, const uint64_t (&pk)[U],
+__device__ __forceinline__ void load_all(const SegArgs& s, const uint32_t (&pk)[U],
                                          RawPack (&raw)[C::K][U]) {
 #pragma unroll
     for (int u = 0; u < U; ++u) raw[k][u] = load_raw<C, k>(s.in[k], pk[u]);
@@ -258,7 +259,7 @@ __device__ __forceinline__ void combine(const RawPack (&raw)[C::K], float (&acc)
 }
 
 template <class C>
-__device__ __forceinline__ void store16(void* base, uint64_t pack, const float (&y)[C::E]) {
+__device__ __forceinline__ void store16(void* base, uint32_t pack, const float (&y)[C::E]) {
     using V = Num<C::W>;
     if constexpr (C::E == 8) {
         u32x4 t;
@@ -273,10 +274,13 @@ __device__ __forceinline__ void store16(void* base, uint64_t pack, const float (
     }
 }
 
+// `has_out` / `has_wire`: which outputs the segment names (the pointers in `s` have
+// been advanced to the tile, so they no longer tell).
 template <class C>
-__device__ __forceinline__ void store_pack(const SegArgs& s, uint64_t pack, const float (&y)[C::E]) {
+__device__ __forceinline__ void store_pack(const SegArgs& s, bool has_out, bool has_wire, uint32_t pack,
+                                           const float (&y)[C::E]) {
     if constexpr (C::W == MCCLX_F32 || C::kOutF32) {
-        if (s.out) {
+        if (has_out) {
             u32x4 t;
 #pragma unroll
             for (int j = 0; j < 4; ++j) t[j] = __float_as_uint(y[j]);
@@ -285,10 +289,10 @@ __device__ __forceinline__ void store_pack(const SegArgs& s, uint64_t pack, cons
     }
     if constexpr (C::W != MCCLX_F32) {
         if constexpr (C::kOutF32) {
-            if (s.wire_out) store16<C>(s.wire_out, pack, y);
+            if (has_wire) store16<C>(s.wire_out, pack, y);
         } else {
-            if (s.out) store16<C>(s.out, pack, y);
-            if (s.wire_out) store16<C>(s.wire_out, pack, y);
+            if (has_out) store16<C>(s.out, pack, y);
+            if (has_wire) store16<C>(s.wire_out, pack, y);
         }
     }
 }
@@ -334,10 +338,12 @@ __device__ __forceinline__ void fold_elem(const SegArgs& s, uint64_t i, float sc
     }
 }
 
-// U packets per lane: all loads first, then arithmetic, then stores.
+// U packets per lane: all loads first, then arithmetic, then stores.  `s` points
+// at the tile's first packet; pk[] are packet indices inside the tile, so every
+// address is a uniform 64-bit base plus a 32-bit lane offset.
 template <class C, int U>
-__device__ __forceinline__ void fold_packs(const SegArgs& s, const uint64_t (&pk)[U], float scale,
-                                           bool has_scale) {
+__device__ __forceinline__ void fold_packs(const SegArgs& s, bool has_out, bool has_wire, const uint32_t (&pk)[U],
+                                           float scale, bool has_scale) {
     RawPack raw[C::K][U];
     load_all<C, 0, U>(s, pk, raw);
 #pragma unroll
@@ -349,7 +355,7 @@ __device__ __forceinline__ void fold_packs(const SegArgs& s, const uint64_t (&pk
         combine<C>(col, acc);
 #pragma unroll
         for (int j = 0; j < C::E; ++j) acc[j] = finish<C>(acc[j], scale, has_scale);
-        store_pack<C>(s, pk[u], acc);
+        store_pack<C>(s, has_out, has_wire, pk[u], acc);
     }
 }
 
@@ -359,59 +365,65 @@ template <class C>
 __device__ __forceinline__ uint32_t head_elems(const SegArgs& s) {
 #if MCCLX_TUNE_PEEL
     const bool wide_out = (C::W == MCCLX_F32 || C::kOutF32) && s.out;
-    const uintptr_t a = reinterpret_cast<uintptr_t>(s.out ? s.out : s.wire_out);
-    const uint32_t es = wide_out ? 4u : 2u;
-    const uint32_t mis = (uint32_t)(a & 127u);
-    const uint64_t h = mis ? (128u - mis) / es : 0u;
-    return (uint32_t)(h < s.count ? h : s.count);
+    const uint32_t a = (uint32_t)reinterpret_cast<uintptr_t>(s.out ? s.out : s.wire_out);
+    const uint32_t mis = a & 127u;
+    const uint32_t h = mis ? (128u - mis) >> (wide_out ? 2 : 1) : 0u;
+    return s.count < h ? (uint32_t)s.count : h;
 #else
     (void)s;
     return 0;
 #endif
 }
 
+// Every pointer of the segment moved `elems` elements on (null outputs become
+// garbage: the caller keeps their presence in flags).
 template <class C>
-__device__ __forceinline__ SegArgs shifted(const SegArgs& s, uint32_t head) {
+__device__ __forceinline__ SegArgs advanced(const SegArgs& s, uint64_t elems) {
     SegArgs t;
+    const uint64_t b2 = elems * 2, b4 = elems * 4;
     const bool out_f32 = (C::W == MCCLX_F32 || C::kOutF32);
-    t.out = s.out ? static_cast<char*>(s.out) + (uint64_t)head * (out_f32 ? 4 : 2) : nullptr;
-    t.wire_out = s.wire_out ? static_cast<char*>(s.wire_out) + (uint64_t)head * 2 : nullptr;
+    t.out = static_cast<char*>(s.out) + (out_f32 ? b4 : b2);
+    t.wire_out = static_cast<char*>(s.wire_out) + b2;
 #pragma unroll
     for (int k = 0; k < MCCLX_MAX_INPUTS; ++k)
-        t.in[k] = (k < C::K) ? static_cast<const char*>(s.in[k]) + (uint64_t)head * (C::in_is_f32(k) ? 4 : 2)
-                             : nullptr;
-    t.count = s.count - head;
+        t.in[k] = (k < C::K) ? static_cast<const char*>(s.in[k]) + (C::in_is_f32(k) ? b4 : b2) : nullptr;
+    t.count = 0;
     return t;
 }
 
-// The block's share of one segment: after the head peel, packets [first, P) in
-// strides of `stride` packets; the block with `do_edges` also runs the head
-// and the sub-packet tail one element per lane.
+// One tile of a segment: after the head peel, the U * kBlock packets from packet
+// `first` on (fewer at the segment's end); the block with `do_edges` also runs
+// the head and the sub-packet tail, one element per lane.  The path to the first
+// load is kept short -- a block lives for about 2 us and eight waves per SIMD
+// share one scalar unit, so every scalar instruction in front of the loads is
+// paid eight times over.
 template <class C>
-__device__ __forceinline__ void fold_segment(const SegArgs& s, float scale, bool has_scale,
-                                             uint64_t first, uint64_t stride, bool do_edges) {
+__device__ __forceinline__ void fold_tile(const SegArgs& s, float scale, bool has_scale, uint64_t first,
+                                          bool do_edges) {
     constexpr int U = C::U;
     const uint32_t tid = threadIdx.x;
     const uint32_t head = head_elems<C>(s);  // < 64 <= kBlock
-    const SegArgs t = shifted<C>(s, head);
-    const uint64_t P = t.count / C::E;
-    for (uint64_t base = first; base < P; base += stride) {
-        if (base + (uint64_t)U * kBlock <= P) {
-            uint64_t pk[U];
+    const uint64_t P = (s.count - head) / C::E;
+    const bool has_out = s.out != nullptr, has_wire = s.wire_out != nullptr;
+    if (first < P) {
+        const SegArgs t = advanced<C>(s, head + first * C::E);
+        const uint64_t left = P - first;
+        if (left >= (uint64_t)U * kBlock) {
+            uint32_t pk[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) pk[u] = base + (uint64_t)u * kBlock + tid;
-            fold_packs<C, U>(t, pk, scale, has_scale);
+            for (int u = 0; u < U; ++u) pk[u] = (uint32_t)u * kBlock + tid;
+            fold_packs<C, U>(t, has_out, has_wire, pk, scale, has_scale);
         } else {
-            for (uint64_t p = base + tid; p < P && p < base + (uint64_t)U * kBlock; p += kBlock) {
-                uint64_t one[1] = {p};
-                fold_packs<C, 1>(t, one, scale, has_scale);
+            for (uint32_t p = tid; p < (uint32_t)left; p += kBlock) {
+                uint32_t one[1] = {p};
+                fold_packs<C, 1>(t, has_out, has_wire, one, scale, has_scale);
             }
         }
     }
     if (do_edges) {
         if (tid < head) fold_elem<C>(s, tid, scale, has_scale);
-        uint64_t i = P * C::E + tid;  // fewer than E <= 8 elements remain
-        if (i < t.count) fold_elem<C>(t, i, scale, has_scale);
+        const uint64_t i = head + P * C::E + tid;  // fewer than E <= 8 elements remain
+        if (i < s.count) fold_elem<C>(s, i, scale, has_scale);
     }
 }
 
@@ -459,10 +471,11 @@ __device__ __forceinline__ void fold_few_body(const FewArgs& a) {
     // workgroups go to the XCDs round robin: block b runs on XCD b % N
     const uint32_t per = grid / MCCLX_TUNE_XCD;  // the grid is a multiple of N
     const uint32_t tile = (blockIdx.x % MCCLX_TUNE_XCD) * per + blockIdx.x / MCCLX_TUNE_XCD;
-    fold_segment<C>(s, scale, has_scale != 0, (uint64_t)tile * span, ~0ull >> 1, tile == 0);
+    fold_tile<C>(s, scale, has_scale != 0, (uint64_t)tile * span, tile == 0);
 #else
-    fold_segment<C>(s, scale, has_scale != 0, (uint64_t)blockIdx.x * span, (uint64_t)grid * span,
-                    blockIdx.x == 0);
+    // one tile per block, no loop: the launch sizes the grid to the longest segment
+    (void)grid;
+    fold_tile<C>(s, scale, has_scale != 0, (uint64_t)blockIdx.x * span, blockIdx.x == 0);
 #endif
 #if MCCLX_TUNE_TIMELINE
     if (a.timeline && threadIdx.x == 0) {
@@ -540,7 +553,7 @@ __device__ __forceinline__ void fold_table_body(const TableArgs& a) {
         for (int k = 0; k < MCCLX_MAX_INPUTS; ++k) s.in[k] = (k < C::K) ? uniptr(d->in[k]) : nullptr;
         s.count = uni64(d->count);
         // one tile: packets [tile*span, tile*span + span); tile 0 also owns the tail
-        fold_segment<C>(s, a.scale, a.has_scale != 0, (uint64_t)tile * span, ~0ull >> 1, tile == 0);
+        fold_tile<C>(s, a.scale, a.has_scale != 0, (uint64_t)tile * span, tile == 0);
     }
 }
 
@@ -568,6 +581,15 @@ extern "C" MCCLX_API void mcclx_tune_timeline(void* device_buf, uint64_t slots, 
 }
 #endif
 
+#ifdef MCCLX_TUNE_MINIMAL
+static size_t wide_lds_bytes() {  // tuning: dynamic LDS reserved per block of a wide fold, to cap blocks per CU
+    static const size_t v = [] { const char* e = getenv("MCCLX_WIDE_LDS"); return e ? (size_t)atol(e) : 0; }();
+    return v;
+}
+#else
+static constexpr size_t wide_lds_bytes() { return 0; }
+#endif
+
 template <class C>
 static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
     const uint64_t span = (uint64_t)C::U * kBlock * C::E;  // elements per block iteration
@@ -584,10 +606,9 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
         uint64_t maxc = 0;
         for (int i = 0; i < a.nseg; ++i) maxc = a.seg[i].count > maxc ? a.seg[i].count : maxc;
         if (maxc == 0) return hipSuccess;
+        // one block per tile of the longest segment (the by-value kernel does not loop)
         uint64_t gx = (maxc + span - 1) / span;
-        uint64_t cap = lp.max_blocks / (uint32_t)a.nseg;
-        if (cap < 1) cap = 1;
-        if (gx > cap) gx = cap;
+        if (gx >> 31) return hipErrorInvalidValue;
 #if MCCLX_TUNE_XCD
         gx = (gx + MCCLX_TUNE_XCD - 1) / MCCLX_TUNE_XCD * MCCLX_TUNE_XCD;
 #endif
@@ -597,7 +618,7 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
         if constexpr (kLightPlan<C>)
             fold_few_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(kBlock), 0, st>>>(a);
         else
-            fold_few_wide_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(kBlock), 0, st>>>(a);
+            fold_few_wide_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(kBlock), wide_lds_bytes(), st>>>(a);
     }
     return hipGetLastError();
 }
