@@ -38,6 +38,9 @@ struct Contribution {
     int wire_bf16 = 0;
     int root = 0;
     void* stream = nullptr;        // the rank's producer/consumer HIP stream
+    void* work = nullptr;          // the rank's completion object, when the leader (or a later
+                                   // launch) settles it instead of the rank itself
+    int async = 0;                 // allreduce: event-based completion asked for (ranks must agree)
     std::vector<uint64_t> in_off;  // all-to-all: byte offsets (or sizes) of what goes to each peer
     std::vector<uint64_t> out_off; // all-to-all: byte offsets (or sizes) of what comes from each peer
     std::string error;             // set when this rank failed its own argument checks: the

@@ -4,8 +4,10 @@
 #include <c10/hip/HIPStream.h>
 
 #include <algorithm>
+#include <atomic>
 #include <condition_variable>
 #include <cstdlib>
+#include <deque>
 #include <cstring>
 #include <functional>
 #include <map>
@@ -116,13 +118,110 @@ struct ProcessGroupMCCL::Shared {
     uint64_t graph_hits = 0;
     bool graphs_enabled = true;
 
+    // Event-based completion (MCCL_ALLREDUCE_ASYNC=1).  An allreduce of the group
+    // becomes a Bucket; it is launched at once when the reduce queue is idle and
+    // parked otherwise, and everything parked goes out together -- one launch per
+    // phase for all of it -- as soon as the launch in flight has finished (or a
+    // rank waits on one of the parked Works).  A worker thread waits for each
+    // launch's completion ticket and settles the ranks' Works.
+    struct Bucket {
+        std::vector<mcclx_replay> reps;
+        std::vector<std::vector<void*>> ptrs;  // reps[i].tensors points into ptrs[i]
+        at::Tensor workspace;                  // wire copies / recv scratch of this call
+        std::vector<c10::intrusive_ptr<WorkMCCL>> works;  // one per rank
+        std::atomic<bool> launched{false};
+    };
+    std::mutex amu;
+    std::deque<std::shared_ptr<Bucket>> parked;
+    uint64_t inflight_ticket = 0;              // ticket of the newest launch
+    std::atomic<uint64_t> finished_ticket{0};  // newest ticket the completer has seen complete
+    bool flush_scheduled = false;
+    std::unique_ptr<Progress> completer;
+    std::atomic<uint64_t> async_launches{0}, async_buckets{0};
+
     Shared() {
         const char* e = std::getenv("MCCL_GRAPH_CACHE");
         graphs_enabled = !(e && e[0] == '0');
     }
     ~Shared() {
+        if (completer) completer->shutdown();  // settles what is still in flight
         drop_graphs();
         if (ctx) mcclx_destroy(ctx);
+    }
+
+    // Caller holds amu.  Issues the buckets as ONE list replay and hands their
+    // Works to the completer.
+    void launch_locked(std::vector<std::shared_ptr<Bucket>> buckets) {
+        std::vector<mcclx_replay> all;
+        for (auto& b : buckets) all.insert(all.end(), b->reps.begin(), b->reps.end());
+        std::exception_ptr err;
+        uint64_t ticket = 0;
+        try {
+            check_rc(mcclx_allreduce_replay_many(ctx, all.data(), static_cast<uint32_t>(all.size())));
+            check_rc(mcclx_event_record(ctx, &ticket));
+        } catch (...) {
+            err = std::current_exception();
+        }
+        for (auto& b : buckets) b->launched = true;
+        if (err) {
+            for (auto& b : buckets)
+                for (auto& w : b->works) w->finishWithException(err);
+            std::rethrow_exception(err);
+        }
+        inflight_ticket = ticket;
+        ++async_launches;
+        async_buckets += buckets.size();
+        if (!completer) completer = std::make_unique<Progress>();
+        mcclx_ctx* c = ctx;
+        completer->submit([this, c, ticket, buckets = std::move(buckets)]() mutable {
+            std::exception_ptr failure;
+            try {
+                check_rc(mcclx_event_wait(c, ticket));
+            } catch (...) {
+                failure = std::current_exception();
+            }
+            finished_ticket.store(ticket);
+            for (auto& b : buckets)
+                for (auto& w : b->works) {
+                    if (failure)
+                        w->finishWithException(failure);
+                    else
+                        w->finish();
+                }
+            buckets.clear();  // workspaces go back to the allocator only now
+        });
+    }
+
+    // Is the newest launch still running?  Answered from what the completer has seen,
+    // not by polling the event: the completer is blocked in a wait on that very event,
+    // and a query from another thread would block with it.
+    bool queue_busy_locked() const { return inflight_ticket != finished_ticket.load(); }
+
+    void submit_bucket(std::shared_ptr<Bucket> b) {
+        std::lock_guard<std::mutex> lk(amu);
+        if (parked.empty() && !queue_busy_locked()) {
+            launch_locked({std::move(b)});
+            return;
+        }
+        parked.push_back(std::move(b));
+        if (!flush_scheduled) {
+            flush_scheduled = true;
+            // runs behind the completion wait of the launch in flight
+            completer->submit([this] { flush_parked(); });
+        }
+    }
+
+    void flush_parked() {
+        std::lock_guard<std::mutex> lk(amu);
+        flush_scheduled = false;
+        if (parked.empty()) return;
+        std::vector<std::shared_ptr<Bucket>> go(parked.begin(), parked.end());
+        parked.clear();
+        try {
+            launch_locked(std::move(go));
+        } catch (...) {
+            // the Works carry the error
+        }
     }
     void drop_graphs() {
         for (auto& kv : graphs)
@@ -254,6 +353,11 @@ ProcessGroupMCCL::~ProcessGroupMCCL() {
 }
 
 uint64_t ProcessGroupMCCL::graphHits() const { return shared_ ? shared_->graph_hits : 0; }
+std::pair<uint64_t, uint64_t> ProcessGroupMCCL::asyncStats() const {
+    if (!shared_) return {0, 0};
+    return {shared_->async_launches.load(), shared_->async_buckets.load()};
+}
+uint64_t ProcessGroupMCCL::launchCount() const { return ctx_ ? mcclx_launch_count(ctx_) : 0; }
 
 void* ProcessGroupMCCL::my_stream() const {
     return static_cast<void*>(c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(device_)).stream());
@@ -349,54 +453,78 @@ int64_t env_tree_below() {
 
 }  // namespace
 
+namespace {
+bool env_async_allreduce() {
+    const char* e = std::getenv("MCCL_ALLREDUCE_ASYNC");  // re-read on every call, like the other knobs
+    return e && e[0] == '1';
+}
+}  // namespace
+
 c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tensor>& tensors,
                                                            const c10d::AllreduceOptions& opts) {
     if (getSize() == 1) return make_completed(c10d::OpType::ALLREDUCE, tensors, "mccl:allreduce");
-    MCCL_CHECK(!tensors.empty(), "allreduce: empty tensor list");
-    const int op = reduce_op_code(opts.reduceOp);
     const int world = getSize();
-    const bool wire = env_wire_bf16();
-    const char* env_alg = std::getenv("MCCL_ALLREDUCE_ALGO");
-    const int64_t tree_below = env_tree_below();
+    const bool async = env_async_allreduce();
+    c10::intrusive_ptr<WorkMCCL> work;
+    if (async) work = c10::make_intrusive<WorkMCCL>(c10d::OpType::ALLREDUCE, tensors, "mccl:allreduce");
 
+    // A rank whose own checks fail still goes to the meeting point, carrying the
+    // message, so that the whole group fails at once instead of waiting for it.
     Contribution c;
-    c.kind = K_ALLREDUCE;
-    c.op = op;
-    c.wire_bf16 = wire ? 1 : 0;
-    c.stream = my_stream();
-    for (auto& t : tensors) {
-        check_gpu_(t, "allreduce");
-        const int dt = need_reduce_dtype(t, "allreduce");
-        MCCL_CHECK(t.numel() > 0, "MCCL does not accept empty tensors");  // TensorChecks.hpp:31-34
-        const bool use_wire = wire && dt == MCCLX_F32;  // :131
-        const uint64_t bytes = static_cast<uint64_t>(t.numel()) * (use_wire ? 2u : t.element_size());
-        c.dst.push_back(t.data_ptr());
-        c.numel.push_back(static_cast<uint64_t>(t.numel()));
-        c.dtype.push_back(dt);
-        c.algo.push_back(mcclx_select_algo(env_alg, tree_below, bytes, t.numel(), world));  // :134-145
+    try {
+        MCCL_CHECK(!tensors.empty(), "allreduce: empty tensor list");
+        const int op = reduce_op_code(opts.reduceOp);
+        const bool wire = env_wire_bf16();
+        const char* env_alg = std::getenv("MCCL_ALLREDUCE_ALGO");
+        const int64_t tree_below = env_tree_below();
+        c.op = op;
+        c.wire_bf16 = wire ? 1 : 0;
+        for (auto& t : tensors) {
+            check_gpu_(t, "allreduce");
+            const int dt = need_reduce_dtype(t, "allreduce");
+            MCCL_CHECK(t.numel() > 0, "MCCL does not accept empty tensors");  // TensorChecks.hpp:31-34
+            const bool use_wire = wire && dt == MCCLX_F32;  // :131
+            const uint64_t bytes = static_cast<uint64_t>(t.numel()) * (use_wire ? 2u : t.element_size());
+            c.dst.push_back(t.data_ptr());
+            c.numel.push_back(static_cast<uint64_t>(t.numel()));
+            c.dtype.push_back(dt);
+            c.algo.push_back(mcclx_select_algo(env_alg, tree_below, bytes, t.numel(), world));  // :134-145
+        }
+        last_algo_ = c.algo.back();
+        MCCL_DEBUG("rank %d allreduce: %zu tensor(s), first numel %llu, op %d, algo %d, wire %s%s", getRank(),
+                   tensors.size(), (unsigned long long)c.numel[0], op, last_algo_, wire ? "bf16" : "native",
+                   async ? ", event-based completion" : "");
+    } catch (const std::exception& e) {
+        c = Contribution{};
+        c.error = e.what();
     }
-    last_algo_ = c.algo.back();
-    MCCL_DEBUG("rank %d allreduce: %zu tensor(s), first numel %llu, op %d, algo %d, wire %s", getRank(), tensors.size(),
-               (unsigned long long)c.numel[0], op, last_algo_, wire ? "bf16" : "native");
+    c.kind = K_ALLREDUCE;
+    c.stream = my_stream();
+    c.async = async ? 1 : 0;
+    c.work = work.get();
     flush_engine_();
 
     auto shared = shared_;
-    // The allreduce is synchronous, as in the reference (ProcessGroupMCCL.cpp:170-185):
-    // when it returns, every rank's tensor holds the result and the queue is drained.
-    meet(std::move(c), [shared, world](const std::vector<Contribution>& all) {
+    const int device = device_;
+    meet(std::move(c), [shared, world, device](const std::vector<Contribution>& all) {
         mcclx_ctx* ctx = shared->ctx;
         const size_t nt = all[0].dst.size();
+        const bool async = all[0].async != 0;
         for (int r = 0; r < world; ++r) {
             MCCL_CHECK(all[r].dst.size() == nt, "allreduce: ranks passed different numbers of tensors");
             MCCL_CHECK(all[r].op == all[0].op && all[r].wire_bf16 == all[0].wire_bf16,
                        "allreduce: ranks disagree on the reduce op or MCCL_WIRE_DTYPE");
+            MCCL_CHECK((all[r].async != 0) == async, "allreduce: ranks disagree on MCCL_ALLREDUCE_ASYNC");
             check_rc(mcclx_queue_wait_stream(ctx, all[r].stream));  // mps_stream_sync, :172
         }
         // one replay per tensor of the list; the reference runs them one after another
         // (ProcessGroupMCCL.cpp:122-168), here a list is issued together so that
         // entries sharing a plan need one launch per phase for all of them
-        std::vector<std::vector<void*>> ptrs(nt, std::vector<void*>(static_cast<size_t>(world)));
-        std::vector<mcclx_replay> reps(nt);
+        auto bucket = std::make_shared<Shared::Bucket>();
+        auto& ptrs = bucket->ptrs;
+        auto& reps = bucket->reps;
+        ptrs.assign(nt, std::vector<void*>(static_cast<size_t>(world)));
+        reps.resize(nt);
         std::vector<uint64_t> need(nt), offset(nt);
         uint64_t total = 0;
         for (size_t i = 0; i < nt; ++i) {
@@ -425,17 +553,55 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
             offset[i] = total;
             total += need[i];
         }
-        char* ws = static_cast<char*>(shared->workspace(total));
+        char* ws = nullptr;
+        if (async && total) {
+            // several calls may be in flight: each keeps a workspace of its own until it has finished
+            bucket->workspace = at::empty({static_cast<int64_t>(total + 256)},
+                                          at::TensorOptions().dtype(at::kByte).device(at::kCUDA, device));
+            order_after_allocator(ctx, device);
+            auto p = reinterpret_cast<uintptr_t>(bucket->workspace.data_ptr());
+            ws = reinterpret_cast<char*>((p + 255) / 256 * 256);
+        } else {
+            ws = static_cast<char*>(shared->workspace(total));
+        }
         for (size_t i = 0; i < nt; ++i) {
             reps[i].workspace = need[i] ? ws + offset[i] : nullptr;
             reps[i].workspace_bytes = need[i];
         }
+        if (async) {
+            for (int r = 0; r < world; ++r) {
+                MCCL_CHECK(all[r].work != nullptr, "allreduce: a rank arrived without its Work");
+                bucket->works.push_back(
+                    c10::intrusive_ptr<WorkMCCL>::reclaim_copy(static_cast<WorkMCCL*>(all[r].work)));
+            }
+            // wait() on any rank's Work: make sure the launch is out, then let the
+            // rank's current stream wait for the queue on the device
+            // (weak references: a Work may outlive the group, and the last Work of a launch is
+            // released on the completer thread, which must never be the one to tear the group down)
+            std::weak_ptr<Shared::Bucket> weak = bucket;
+            std::weak_ptr<Shared> weak_shared = shared;
+            for (auto& w : bucket->works)
+                w->setWaitHook([weak_shared, weak, device] {
+                    auto sh = weak_shared.lock();
+                    if (!sh) return;  // the group is gone: its destructor has drained the queue
+                    if (auto b = weak.lock())
+                        if (!b->launched) sh->flush_parked();
+                    check_rc(mcclx_stream_wait_queue(
+                        sh->ctx,
+                        static_cast<void*>(c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(device)).stream())));
+                });
+            shared->submit_bucket(bucket);
+            return;
+        }
+        // The reference's allreduce is synchronous (ProcessGroupMCCL.cpp:170-185): when
+        // it returns, every rank's tensor holds the result and the queue is drained.
         if (nt == 1)
             shared->allreduce(reps[0]);  // a single bucket: recorded and replayed when it comes again
         else
             check_rc(mcclx_allreduce_replay_many(ctx, reps.data(), static_cast<uint32_t>(nt)));
         check_rc(mcclx_queue_drain(ctx));  // mccl_queue_drain, :178
     });
+    if (async) return work;
     return make_completed(c10d::OpType::ALLREDUCE, tensors, "mccl:allreduce");
 }
 

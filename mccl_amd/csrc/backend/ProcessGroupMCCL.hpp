@@ -21,6 +21,7 @@
 #include <functional>
 #include <memory>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "mcclx.h"
@@ -69,6 +70,10 @@ public:
     int lastAlgo() const { return last_algo_; }
     // Allreduces of this rank's group that were replayed from a recorded graph, for tests.
     uint64_t graphHits() const;
+    // Event-based allreduces of this rank's group: (launches issued, buckets they carried), and the
+    // kernel launches the group's reduce queue has issued so far; for tests and the benchmark.
+    std::pair<uint64_t, uint64_t> asyncStats() const;
+    uint64_t launchCount() const;
 
 private:
     struct Shared;  // reduce queue, scratch and recorded graphs shared by the ranks of one mesh

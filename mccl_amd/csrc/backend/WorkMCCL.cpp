@@ -58,6 +58,12 @@ void WorkMCCL::finishWithException(std::exception_ptr error) {
 }
 
 bool WorkMCCL::wait(std::chrono::milliseconds timeout) {
+    if (on_wait_) {
+        on_wait_();  // stream-ordered: the caller's stream now waits for the result on the device
+        std::lock_guard<std::mutex> lk(mu_);
+        if (state_ == State::Failed) std::rethrow_exception(error_);
+        return true;
+    }
     std::unique_lock<std::mutex> lk(mu_);
     const auto settled = [this] { return state_ != State::Pending; };
     if (timeout == kNoTimeout)

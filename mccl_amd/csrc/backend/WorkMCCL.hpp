@@ -31,6 +31,12 @@ public:
 
     // -- what the issuing side calls (the engine thread, or the caller's thread for allreduce)
     void setSyncCallback(std::function<void()> before_done) { before_done_ = std::move(before_done); }
+    // Event-based completion: with a wait hook, wait() does not block the host until
+    // the Work is settled.  It runs the hook -- which makes the caller's stream wait,
+    // on the device, for the reduce queue -- and returns; the Work and its Future
+    // settle later, when the device has finished.  A Work that has already failed
+    // still rethrows from wait().
+    void setWaitHook(std::function<void()> on_wait) { on_wait_ = std::move(on_wait); }
     void finish();
     void finishWithException(std::exception_ptr error);
 
@@ -51,6 +57,7 @@ private:
     std::vector<at::Tensor> outputs_;
     c10::intrusive_ptr<c10::ivalue::Future> future_;
     std::function<void()> before_done_;
+    std::function<void()> on_wait_;
 
     mutable std::mutex mu_;
     std::condition_variable settled_cv_;

@@ -182,6 +182,15 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         return p ? p->graphHits() : uint64_t(0);
     });
 
+    m.def("_async_stats", [](const c10::intrusive_ptr<c10d::Backend>& pg) {
+        auto* p = dynamic_cast<mccl::ProcessGroupMCCL*>(pg.get());
+        return p ? p->asyncStats() : std::pair<uint64_t, uint64_t>(0, 0);
+    });
+    m.def("_launch_count", [](const c10::intrusive_ptr<c10d::Backend>& pg) {
+        auto* p = dynamic_cast<mccl::ProcessGroupMCCL*>(pg.get());
+        return p ? p->launchCount() : uint64_t(0);
+    });
+
     m.def("_test_progress_order", &progress_order, py::arg("n"), py::arg("throw_mask") = 0,
           py::arg("use_destructor") = false, py::call_guard<py::gil_scoped_release>());
     m.def("_test_log", [](int level, const std::string& text) {

@@ -78,7 +78,11 @@ struct mcclx_ctx {
     bool batch_active = false;
     std::string batch_label;
     std::mutex mu;
-    std::unordered_map<uint64_t, hipEvent_t> tickets;
+    struct Ticket {
+        hipEvent_t ev = nullptr;
+        int waiters = 0;  // threads inside hipEventSynchronize on `ev`
+    };
+    std::unordered_map<uint64_t, Ticket> tickets;
     std::vector<hipEvent_t> free_events;
     uint64_t next_ticket = 1;
     hipEvent_t t0 = nullptr, t1 = nullptr;
@@ -323,8 +327,7 @@ int ensure_slot(mcclx_ctx* ctx, TableSlot& sl, size_t need) {
 
 // Puts a descriptor table where a kernel can read it (caller holds ctx->mu).
 // Outside a recording: the next slot of the pinned staging ring, copied to its
-// device twin on the queue; `*slot` must be handed to table_launched() after
-// the launch.  While recording: the launch needs a table that outlives this
+// device twin on the queue (`*slot` names it).  While recording: the launch needs a table that outlives this
 // call, so it gets its own device buffer, filled now with a blocking copy
 // (outside the recording) and owned by the graph; `*slot` stays null.
 int stage_table(mcclx_ctx* ctx, const void* bytes, size_t nbytes, void** dev, TableSlot** slot) {
@@ -345,21 +348,28 @@ int stage_table(mcclx_ctx* ctx, const void* bytes, size_t nbytes, void** dev, Ta
         *dev = d;
         return MCCLX_OK;
     }
+    // The queue may be a stream the caller owns (mcclx_init_on_stream) and is recording
+    // into a graph of its own: a table upload recorded there would replay whatever the
+    // staging ring holds at that time.  Such callers record through mcclx_graph_begin or
+    // use the allocation-free entry point, whose table travels in kernel arguments.
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(ctx->stream, &cap) != hipSuccess) (void)hipGetLastError();
+    if (cap != hipStreamCaptureStatusNone)
+        return fail(MCCLX_ERR_STATE,
+                    "a launch with a descriptor table cannot be recorded by a stream capture the library did not "
+                    "start: record with mcclx_graph_begin, or use mcclx_fold_batched_noalloc");
     TableSlot& sl = ctx->slots[ctx->next_slot];
     ctx->next_slot = (ctx->next_slot + 1) % kTableSlots;
     if (int rc = ensure_slot(ctx, sl, nbytes)) return rc;
     memcpy(sl.host, bytes, nbytes);
     HIP_TRY(hipMemcpyAsync(sl.dev, sl.host, nbytes, hipMemcpyHostToDevice, ctx->stream));
+    // The slot's pinned half is busy until this copy has run; its device half is only
+    // touched on the queue, whose order keeps the next upload behind the launch that
+    // reads this one.  Recorded here, so that no exit path of the caller can skip it.
+    HIP_TRY(hipEventRecord(sl.done, ctx->stream));
+    sl.pending = true;
     *dev = sl.dev;
     *slot = &sl;
-    return MCCLX_OK;
-}
-
-// The launch that reads the staged table has been issued: the slot is busy until it ends.
-int table_launched(mcclx_ctx* ctx, TableSlot* slot) {
-    if (!slot) return MCCLX_OK;
-    HIP_TRY(hipEventRecord(slot->done, ctx->stream));
-    slot->pending = true;
     return MCCLX_OK;
 }
 
@@ -454,7 +464,7 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
     hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
     if (e != hipSuccess) return launch_error(e, key);
     ++ctx->launches;
-    return table_launched(ctx, slot);
+    return MCCLX_OK;
 }
 
 int make_ctx(int device, hipStream_t borrowed, bool borrow, mcclx_ctx** out) {
@@ -534,7 +544,7 @@ int mcclx_destroy(mcclx_ctx* ctx) {
     if (!ctx) return MCCLX_OK;
     DeviceGuard guard(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
-    for (auto& kv : ctx->tickets) (void)hipEventDestroy(kv.second);
+    for (auto& kv : ctx->tickets) (void)hipEventDestroy(kv.second.ev);
     for (auto ev : ctx->free_events) (void)hipEventDestroy(ev);
     for (auto ev : ctx->xev)
         if (ev) (void)hipEventDestroy(ev);
@@ -795,7 +805,7 @@ int mcclx_copy_batched(mcclx_ctx* ctx, const mcclx_copy_desc* descs, uint32_t n)
     hipError_t e = mcclx::launch_copy_many(ctx->stream, t, align, ctx->max_blocks);
     if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "copy_batched launch failed: %s", hipGetErrorString(e));
     ++ctx->launches;
-    return table_launched(ctx, slot);
+    return MCCLX_OK;
 }
 
 int mcclx_batch_begin(mcclx_ctx* ctx, const char* label) {
@@ -856,7 +866,7 @@ int mcclx_event_record(mcclx_ctx* ctx, uint64_t* ticket) {
     if (int rc = get_event(ctx, &ev)) return rc;
     HIP_TRY(hipEventRecord(ev, ctx->stream));
     *ticket = ctx->next_ticket++;
-    ctx->tickets[*ticket] = ev;
+    ctx->tickets[*ticket].ev = ev;
     return MCCLX_OK;
 }
 
@@ -870,7 +880,7 @@ int mcclx_event_query(mcclx_ctx* ctx, uint64_t ticket, int* done) {
         *done = 1;
         return MCCLX_OK;
     }
-    hipError_t e = hipEventQuery(it->second);
+    hipError_t e = hipEventQuery(it->second.ev);
     if (e == hipSuccess) {
         *done = 1;
     } else if (e == hipErrorNotReady) {
@@ -891,15 +901,19 @@ int mcclx_event_wait(mcclx_ctx* ctx, uint64_t ticket) {
         auto it = ctx->tickets.find(ticket);
         if (it == ctx->tickets.end()) {
             if (ticket >= ctx->next_ticket) return fail(MCCLX_ERR_INVALID, "unknown ticket");
-            return MCCLX_OK;
+            return MCCLX_OK;  // waited for before: complete
         }
-        ev = it->second;
-        ctx->tickets.erase(it);
+        ev = it->second.ev;
+        ++it->second.waiters;  // the ticket stays known (and pollable) until the wait is over
     }
     hipError_t e = hipEventSynchronize(ev);
     {
         std::lock_guard<std::mutex> lk(ctx->mu);
-        ctx->free_events.push_back(ev);
+        auto it = ctx->tickets.find(ticket);
+        if (it != ctx->tickets.end() && --it->second.waiters == 0) {
+            ctx->free_events.push_back(ev);  // the last waiter retires the ticket
+            ctx->tickets.erase(it);
+        }
     }
     if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "hipEventSynchronize failed: %s", hipGetErrorString(e));
     return MCCLX_OK;
@@ -951,6 +965,7 @@ int mcclx_graph_end(mcclx_ctx* ctx, mcclx_graph** out) {
     // stage the launch's kernel arguments on the device now rather than during the first replay
     if (e == hipSuccess) e = hipGraphUpload(g->exec, ctx->stream);
     if (e != hipSuccess) {
+        if (g->exec) (void)hipGraphExecDestroy(g->exec);
         if (g->graph) (void)hipGraphDestroy(g->graph);
         for (void* t : g->tables) (void)hipFree(t);
         delete g;

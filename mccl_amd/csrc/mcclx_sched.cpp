@@ -508,6 +508,28 @@ int run_stepwise(mcclx_ctx* ctx, const mcclx_replay* r) {
     return replay_stepwise(ctx, &s, Ls);
 }
 
+// Byte ranges one replay reads or writes: its rank tensors and its workspace.
+struct Range {
+    uintptr_t lo, hi;
+};
+void ranges_of(const mcclx_replay* r, std::vector<Range>& out) {
+    const uint64_t tb = r->numel * esize(r->dtype);
+    for (int i = 0; i < r->world; ++i) {
+        const uintptr_t p = reinterpret_cast<uintptr_t>(r->tensors[i]);
+        out.push_back(Range{p, p + tb});
+    }
+    if (r->workspace && r->workspace_bytes) {
+        const uintptr_t p = reinterpret_cast<uintptr_t>(r->workspace);
+        out.push_back(Range{p, p + r->workspace_bytes});
+    }
+}
+bool overlaps(const std::vector<Range>& a, const std::vector<Range>& b) {
+    for (const Range& x : a)
+        for (const Range& y : b)
+            if (x.lo < y.hi && y.lo < x.hi) return true;
+    return false;
+}
+
 // Same plan for every phase?
 bool same_plan(const mcclx_replay* a, const mcclx_replay* b) {
     return a->world == b->world && a->algo == b->algo && a->op == b->op && a->dtype == b->dtype &&
@@ -571,15 +593,24 @@ int mcclx_allreduce_replay_many(mcclx_ctx* ctx, const mcclx_replay* rs, uint32_t
             ++i;
             continue;
         }
-        // gather the run of fused replays that share this one's plan
+        // Gather the run of fused replays that share this one's plan.  The entries of a
+        // run are issued phase by phase, not one after another, so a run also ends at an
+        // entry that touches memory an earlier entry of the run touches (a tensor named
+        // twice, overlapping workspaces): that entry starts a run of its own and sees the
+        // earlier result, as in the reference's one-by-one loop (ProcessGroupMCCL.cpp:173-177).
         Phases ph;
         const mcclx_replay* first = &rs[i];
+        std::vector<Range> taken, mine;
         while (i < n) {
             if (&rs[i] != first) {
                 if (!same_plan(first, &rs[i])) break;
                 TRY(check_replay(ctx, &rs[i], &fused, &nothing));
                 if (!fused || nothing) break;
             }
+            mine.clear();
+            ranges_of(&rs[i], mine);
+            if (overlaps(taken, mine)) break;
+            taken.insert(taken.end(), mine.begin(), mine.end());
             collect_fused(&rs[i], layout_of(&rs[i]), ph);
             ++i;
         }

@@ -297,6 +297,96 @@ def test_error_paths(CX, U):
         assert m["after"] == [3.0] * 5
 
 
+def test_divergent_argument_error_fails_every_rank_at_once(CX):
+    """One rank passes a tensor its own checks refuse (CPU, non-contiguous, empty): that rank still
+    goes to the meeting point, so its peers fail with its message instead of waiting for the
+    group's timeout (20 s here)."""
+    import time
+    world = 3
+    bad = {0: lambda: torch.ones(8), 1: lambda: torch.ones(4, 4, device="cuda").t(),
+           2: lambda: torch.ones(0, device="cuda")}
+
+    def fn(r, pg):
+        msgs, took = [], []
+        for culprit in range(world):
+            t = bad[culprit]() if r == culprit else torch.ones(8, device="cuda")
+            t0 = time.monotonic()
+            try:
+                pg.allreduce([t])
+                msgs.append("no error")
+            except RuntimeError as e:
+                msgs.append(str(e))
+            took.append(time.monotonic() - t0)
+        ok = torch.full((5,), float(r + 1), device="cuda")
+        pg.allreduce([ok]).wait()               # the group is still usable
+        return msgs, took, ok.cpu().tolist()
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for r, (msgs, took, ok) in enumerate(out):
+        assert "GPU-only; got CPU tensor" in msgs[0] and "must be contiguous" in msgs[1] and "empty tensors" in msgs[2]
+        for culprit in range(world):
+            if r != culprit:
+                assert f"(raised on rank {culprit})" in msgs[culprit]
+        assert max(took) < 5.0, took
+        assert ok == [6.0] * 5
+
+
+def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypatch):
+    """MCCL_ALLREDUCE_ASYNC=1: allreduce returns a pending Work, wait() orders the caller's
+    stream after the reduce queue without blocking the host, the Future settles from the
+    completion ticket, and buckets issued while an earlier one is still running go out
+    together (one launch per phase for all of them).  Results are the oracle's, bit for bit."""
+    monkeypatch.setenv("MCCL_ALLREDUCE_ASYNC", "1")
+    monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "butterfly")
+    monkeypatch.setenv("MCCL_WIRE_DTYPE", "bf16")
+    world = 3
+    sizes = [6_553_600, 1_000_003, 70_001, 1_000_003]
+    rng = np.random.default_rng(31)
+    xs = [[(rng.standard_normal(n) * 1e-3).astype(np.float32) for _ in range(world)] for n in sizes]
+
+    def fn(r, pg):
+        ts = [U.to_dev(x[r], F32) for x in xs]
+        big = torch.empty(1 << 30, dtype=torch.uint8, device="cuda") if r == 0 else None
+        torch.cuda.current_stream().synchronize()
+        before = (CX._async_stats(pg), CX._launch_count(pg))
+        if r == 0:
+            # the rank's stream is still busy (a backward pass would be): some 25 ms of copies in
+            # front of the first bucket, so the later buckets find the reduce queue occupied
+            for _ in range(100):
+                big[: 1 << 29].copy_(big[1 << 29:])
+        works = []
+        for t in ts:
+            o = dist.AllreduceOptions(); o.reduceOp = dist.ReduceOp.AVG
+            works.append(pg.allreduce([t], o))
+        pending_at_return = [not w.is_completed() for w in works]
+        for w in works:
+            assert w.wait()                       # stream-ordered: does not block until the device is done
+        doubled = [t * 2 for t in ts]             # torch work on this rank's stream, behind the reduction
+        futs = [w.get_future().wait() for w in works]
+        torch.cuda.current_stream().synchronize()
+        assert all(w.is_completed() and w.is_success() for w in works)
+        assert all(f[0].data_ptr() == t.data_ptr() for f, t in zip(futs, ts))
+        after = (CX._async_stats(pg), CX._launch_count(pg))
+        return ts, doubled, pending_at_return, before, after
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for i, n in enumerate(sizes):
+        want = [x.copy() for x in xs[i]]
+        rc, used = orc.pg_allreduce(want, F32, AVG, wire_bf16=True, env_algo="butterfly", threads=orc.max_threads())
+        assert rc == 0 and used == BUTTERFLY
+        for r in range(world):
+            U.assert_same_bits(out[r][0][i], want[r], F32, f"bucket {i} rank {r}")
+            assert torch.equal(out[r][1][i], out[r][0][i] * 2)
+    (l0, b0), k0 = out[0][3]
+    (l1, b1), k1 = out[0][4]
+    assert b1 - b0 == len(sizes)
+    assert l1 - l0 == 2, "the first bucket alone, the three behind it together"
+    assert k1 - k0 == 3 * 2, "a launch of several buckets is encode + fold + cast, once"
+    assert all(all(out[r][2]) for r in range(world)), "a Work was complete when allreduce returned"
+
+
 def test_reference_collective_vectors(CX):
     """tests/collectives/test_allreduce.py:11-28 (128 x value rank+1, all ops, f32/f16/bf16)
     and tests/test_process_group_local.py:162-207 (3 ranks: SUM = 6, AVG = 2)."""

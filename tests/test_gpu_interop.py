@@ -90,3 +90,64 @@ def test_received_bytes_then_reduce_matches_reference_order(env):
     K.hip_reduce_op_view(d_own.data_ptr(), scratch.data_ptr(), L.BF16, n, "sum")
     want = own.copy(); orc.reduce(want, peer, BF16, SUM)
     U.assert_same_bits(d_own, want, BF16, "unstage + reduce")
+
+
+def test_ticket_stays_pollable_while_another_thread_waits(env):
+    """A ticket another thread is waiting on must not read as complete before the device work is."""
+    import threading
+    from mccl_amd import kernels
+    q = kernels.ReduceQueue(0)
+    n = 1 << 30
+    buf = torch.empty(2 * n, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    for _ in range(6):
+        q.copy(buf.data_ptr() + n, buf.data_ptr(), n)      # about 2 ms of queued work
+    ticket = q.record()
+    seen_done_early = []
+    waiter = threading.Thread(target=lambda: q.wait(ticket))
+    waiter.start()
+    while waiter.is_alive():
+        done = q.query(ticket)
+        if done and waiter.is_alive():
+            # complete by the library's word: then the waiter must be about to return
+            waiter.join(1.0)
+            seen_done_early.append(waiter.is_alive())
+    waiter.join()
+    assert not any(seen_done_early)
+    assert q.query(ticket)                                  # retired tickets read as complete
+    q.close()
+
+
+def test_table_launch_refuses_a_capture_it_did_not_start_and_noalloc_records(env):
+    """A context on the caller's stream: while the caller records that stream into a graph, a launch
+    that needs a descriptor table is refused (its staging ring would be replayed stale), and the
+    allocation-free entry point -- kernel launches only -- records and replays correctly."""
+    import ctypes as C
+    from mccl_amd import _lib as L, kernels
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        q = kernels.ReduceQueue(0, on_torch_stream=True)
+        nseg, n = 40, 3001
+        a = torch.arange(nseg * n, dtype=torch.float32, device="cuda")
+        b = torch.ones(nseg * n, dtype=torch.float32, device="cuda")
+        out = torch.zeros_like(a)
+        plan = kernels.make_plan(L.F32, 2)
+        segs = [kernels.make_seg(out.data_ptr() + 4 * n * i, 0, [a.data_ptr() + 4 * n * i, b.data_ptr() + 4 * n * i], n)
+                for i in range(nseg)]
+        arr = (L.Seg * nseg)(*segs)
+        side.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            rc = L.lib().mcclx_fold_batched(q.handle, C.byref(plan), arr, nseg)
+            msg = L.last_error()
+            rc2 = L.lib().mcclx_fold_batched_noalloc(q.handle, C.byref(plan), arr, nseg)
+        assert rc == L.ERR_STATE and "did not start" in msg
+        assert rc2 == L.OK
+        for rep in range(3):
+            out.zero_()
+            b.fill_(float(rep + 1))
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, a + (rep + 1)), rep
+        q.close()

@@ -309,6 +309,28 @@ def test_many_messages_in_one_replay_equal_single_replays(H, U, algo, dtype, wir
             U.assert_same_bits(g[r], want[r], dtype, f"algo {algo} n {n} rank {r}")
 
 
+def test_list_replay_with_a_tensor_named_twice_runs_in_order(H, U):
+    """A list whose entries share memory cannot be issued phase by phase: the second
+    allreduce of the same tensors must see the first one's result, as in the reference's
+    one-by-one loop (ProcessGroupMCCL.cpp:173-177)."""
+    world = 3
+    rng = np.random.default_rng(44)
+    for dtype, wire in ((F32, False), (F32, True), (BF16, False)):
+        a = [U.rand_values(rng, 5003, dtype, scale=1e-2) for _ in range(world)]
+        b = [U.rand_values(rng, 777, dtype, scale=1e-2) for _ in range(world)]
+        da, db = [U.to_dev(x, dtype) for x in a], [U.to_dev(x, dtype) for x in b]
+        H.allreduce_replay_many([da, db, da, da], "sum", BUTTERFLY, wire_bf16=wire)
+        wa, wb = [x.copy() for x in a], [x.copy() for x in b]
+        for bufs, times in ((wa, 3), (wb, 1)):
+            for _ in range(times):
+                rc = orc.allreduce(BUTTERFLY, bufs, dtype, SUM) if not wire else \
+                    orc.pg_allreduce(bufs, dtype, SUM, wire_bf16=True, env_algo="butterfly")[0]
+                assert rc == 0
+        for r in range(world):
+            U.assert_same_bits(da[r], wa[r], dtype, f"tensor reduced three times, rank {r}")
+            U.assert_same_bits(db[r], wb[r], dtype, f"tensor reduced once, rank {r}")
+
+
 def test_copy_batched_many_small_and_a_few_large(K, U):
     rng = np.random.default_rng(3)
     q = K._q(None)
