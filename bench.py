@@ -385,6 +385,100 @@ def timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure,
     print("\n".join(out))
 
 
+def backend_extras(torch, W):
+    """The same work through the c10d surface: N ranks as N threads of this process, each with
+    its own ProcessGroupMCCL.  (a) eight C2 buckets per rank, back to back, synchronous (the
+    reference's behaviour) and with event-based completion; (b) the C3 ring with MCCL_WIRE=host,
+    every chunk crossing the byte transport in pinned host memory."""
+    import datetime
+    import threading
+    import time
+    import torch.distributed as dist
+    from mccl_amd import _C as CX
+    out = {}
+    saved = {k: os.environ.get(k) for k in ("MCCL_ALLREDUCE_ASYNC", "MCCL_ALLREDUCE_ALGO", "MCCL_WIRE_DTYPE", "MCCL_WIRE")}
+
+    def run(world, body):
+        store = dist.HashStore()
+        res, errs = [None] * world, [None] * world
+
+        def go(r):
+            try:
+                torch.cuda.set_device(0)
+                pg = CX._create_process_group_mccl(store, r, world, datetime.timedelta(seconds=120))
+                res[r] = body(r, pg)
+            except BaseException as e:  # noqa: BLE001
+                errs[r] = e
+        ts = [threading.Thread(target=go, args=(r,)) for r in range(world)]
+        [t.start() for t in ts]
+        [t.join() for t in ts]
+        for e in errs:
+            if e is not None:
+                raise e
+        return res
+
+    try:
+        os.environ.update({"MCCL_ALLREDUCE_ALGO": "butterfly", "MCCL_WIRE_DTYPE": "bf16"})
+        os.environ.pop("MCCL_WIRE", None)
+        nb, numel = 8, W.C2["numel"]
+        for mode in ("sync", "async"):
+            if mode == "async":
+                os.environ["MCCL_ALLREDUCE_ASYNC"] = "1"
+            else:
+                os.environ.pop("MCCL_ALLREDUCE_ASYNC", None)
+
+            def buckets(r, pg):
+                ts = [torch.randn(numel, device="cuda") * 1e-3 for _ in range(nb)]
+                opt = dist.AllreduceOptions()
+                opt.reduceOp = dist.ReduceOp.AVG
+                best = 1e9
+                for rep in range(4):          # the first round records, later rounds replay (sync) or coalesce (async)
+                    torch.cuda.synchronize()
+                    pg.barrier().wait()
+                    before = CX._async_stats(pg)
+                    t0 = time.perf_counter()
+                    works = [pg.allreduce([t], opt) for t in ts]
+                    for w in works:
+                        w.wait()
+                    torch.cuda.current_stream().synchronize()
+                    best = min(best, time.perf_counter() - t0)
+                    after = CX._async_stats(pg)
+                return best, after[0] - before[0]
+            res = run(3, buckets)
+            out[f"c2_backend_{mode}_us_per_bucket"] = round(max(b for b, _ in res) / nb * 1e6, 1)
+            if mode == "async":
+                out["c2_backend_async_launches_for_8_buckets"] = int(res[0][1])
+        os.environ.pop("MCCL_ALLREDUCE_ASYNC", None)
+
+        os.environ.update({"MCCL_ALLREDUCE_ALGO": "ring", "MCCL_WIRE": "host"})
+        n3 = W.C3["numel"]
+
+        def c3(r, pg):
+            t = torch.randn(n3, device="cuda") * 1e-4
+            torch.cuda.synchronize()
+            best = None
+            for rep in range(2):
+                pg.barrier().wait()
+                t0 = time.perf_counter()
+                pg.allreduce([t]).wait()
+                wall = time.perf_counter() - t0
+                st = CX._wire_stats(pg)
+                if best is None or st[4] < best[0]:
+                    best = (st[4], st[2], wall)
+            return best
+        res = run(4, c3)
+        out["c3_backend_host_wire_fold_ms_per_rank"] = [round(ms, 2) for ms, _, _ in res]
+        out["c3_backend_host_wire_fold_PCIe_GBps_best_rank"] = round(max(pb / ms / 1e6 for ms, pb, _ in res), 1)
+        out["c3_backend_host_wire_allreduce_wall_ms"] = round(max(w for _, _, w in res) * 1e3, 1)
+    finally:
+        for k, v in saved.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+    return out
+
+
 def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_segs, measure, gbs):
     """Secondary measurements: the other legs of C2 and the other configurations."""
     out = {}
@@ -595,6 +689,13 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
             q.host_free(hptr)
     del t3, w3
 
+    del hbm_segs
+    torch.cuda.empty_cache()
+    try:
+        out.update(backend_extras(torch, W))
+    except Exception as e:
+        out["backend_extras_error"] = f"{type(e).__name__}: {e}"
+
     # C5: reduce_scatter (8-input bf16 fold per rank, per-step rounding) and the allgather copy
     n5, w5 = W.C5["numel"], 8
     ch5 = n5 // w5
@@ -609,7 +710,7 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
         out[f"c5_reduce_scatter_{name}_us"] = round(ms / 5 * 1e3, 1)
         out[f"c5_reduce_scatter_{name}_GBps"] = round(gbs(9 * ch5 * 2 * w5, ms / 5), 1)
     g5 = torch.empty(n5, dtype=torch.bfloat16, device="cuda")
-    ms, _ = measure(lambda i: [q.copy(g5.data_ptr() + 2 * ch5 * p, o5[p].data_ptr(), 2 * ch5) for p in range(w5)], 5, 1)
+    ms, _ = measure(lambda i: q.copy_batched([(g5.data_ptr() + 2 * ch5 * p, o5[p].data_ptr(), 2 * ch5) for p in range(w5)]), 5, 1)
     out["c5_allgather_copy_one_rank_GBps"] = round(gbs(2 * n5 * 2, ms / 5), 1)
     return out
 

@@ -91,7 +91,7 @@ def build(force: bool = True, verbose: bool = False) -> str:
 
 
 BACKEND_DIR = os.path.join(CSRC, "backend")
-BACKEND_SOURCES = ["Progress.cpp", "LocalMesh.cpp", "WorkMCCL.cpp", "ProcessGroupMCCL.cpp", "bindings.cpp"]
+BACKEND_SOURCES = ["Progress.cpp", "LocalMesh.cpp", "WorkMCCL.cpp", "HostWire.cpp", "ProcessGroupMCCL.cpp", "bindings.cpp"]
 
 
 def backend_path() -> str:

@@ -1,6 +1,7 @@
 #include "backend/LocalMesh.hpp"
 
 #include <atomic>
+#include <cstring>
 #include <map>
 #include <unistd.h>
 
@@ -108,6 +109,50 @@ Parcel LocalMesh::take(int src, int dst, std::chrono::milliseconds timeout) {
     Parcel p = std::move(box.front());
     box.pop_front();
     return p;
+}
+
+void LocalMesh::wire_send(int src, int dst, const void* buf, size_t len, std::shared_ptr<void> keep) {
+    MCCL_CHECK(src >= 0 && src < world_ && dst >= 0 && dst < world_ && src != dst, "wire: bad peer");
+    MCCL_CHECK(buf != nullptr || len == 0, "wire: send from a null buffer");
+    WireMessage m;
+    m.len = len;
+    if (keep) {
+        m.data = buf;
+        m.keep = std::move(keep);
+    } else {
+        m.owned.assign(static_cast<const uint8_t*>(buf), static_cast<const uint8_t*>(buf) + len);
+        m.data = m.owned.data();
+    }
+    {
+        std::lock_guard<std::mutex> lk(wire_mu_);
+        auto& q = wires_[static_cast<size_t>(src) * static_cast<size_t>(world_) + static_cast<size_t>(dst)];
+        q.push_back(std::move(m));
+        // `owned` may have moved: its bytes are where the vector's storage is now
+        if (!q.back().keep) q.back().data = q.back().owned.data();
+    }
+    wire_cv_.notify_all();
+}
+
+void LocalMesh::wire_recv(int src, int dst, void* buf, size_t len, std::chrono::milliseconds timeout) {
+    MCCL_CHECK(src >= 0 && src < world_ && dst >= 0 && dst < world_ && src != dst, "wire: bad peer");
+    auto& q = wires_[static_cast<size_t>(src) * static_cast<size_t>(world_) + static_cast<size_t>(dst)];
+    WireMessage m;
+    {
+        std::unique_lock<std::mutex> lk(wire_mu_);
+        auto ready = [&] { return !q.empty(); };
+        if (timeout.count() <= 0) {
+            wire_cv_.wait(lk, ready);
+        } else if (!wire_cv_.wait_for(lk, timeout, ready)) {
+            throw TimeoutError("rank " + std::to_string(dst) + ": no bytes from rank " + std::to_string(src) +
+                               " within " + std::to_string(timeout.count()) + " ms");
+        }
+        m = std::move(q.front());
+        q.pop_front();
+        if (!m.keep) m.data = m.owned.data();
+    }
+    MCCL_CHECK(m.len == len, "wire: rank " + std::to_string(dst) + " expects " + std::to_string(len) +
+                                 " bytes from rank " + std::to_string(src) + ", which sent " + std::to_string(m.len));
+    if (len) std::memcpy(buf, m.data, len);  // the wire's delivery into the receiver's buffer
 }
 
 }  // namespace mccl

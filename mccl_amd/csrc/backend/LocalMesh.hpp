@@ -3,12 +3,19 @@
 //
 // The reference moves peer chunks over blocking TCP sockets between processes.
 // This build runs every rank of a group inside ONE process on ONE GPU (there is
-// no cross-GPU transport here), so "send/recv" degenerates to: every rank
-// publishes where its tensors live, waits until all ranks of the group have
-// reached the same collective, and the last rank to arrive launches the device
-// work for the whole group -- peers' chunks are read in place.  Collectives
-// must be issued in the same order on every rank, exactly as with the
-// reference's FIFO engine (Progress.hpp:12-18).
+// no cross-GPU transport here), and offers the ranks two ways to meet:
+//
+//  * rendezvous: every rank publishes where its tensors live, waits until all
+//    ranks of the group have reached the same collective, and the last rank to
+//    arrive launches the device work for the whole group -- peers' chunks are
+//    read in place (the default path of every collective);
+//  * a byte transport with PeerMesh's own interface, send(peer, buf, len) /
+//    recv(peer, buf, len) on host-addressable memory (LocalPeer below): one
+//    FIFO per ordered pair of ranks, as a socket per peer gives the reference.
+//    The allreduce's host-wire modes (MCCL_WIRE=host|staged) run over it.
+//
+// Collectives must be issued in the same order on every rank, exactly as with
+// the reference's FIFO engine (Progress.hpp:12-18).
 #pragma once
 
 #include <chrono>
@@ -41,6 +48,7 @@ struct Contribution {
     void* work = nullptr;          // the rank's completion object, when the leader (or a later
                                    // launch) settles it instead of the rank itself
     int async = 0;                 // allreduce: event-based completion asked for (ranks must agree)
+    int transport = 0;             // allreduce: 0 = peers read in place, 1 = pinned host wire, 2 = staged host wire
     std::vector<uint64_t> in_off;  // all-to-all: byte offsets (or sizes) of what goes to each peer
     std::vector<uint64_t> out_off; // all-to-all: byte offsets (or sizes) of what comes from each peer
     std::string error;             // set when this rank failed its own argument checks: the
@@ -58,13 +66,25 @@ struct Parcel {
     std::shared_ptr<void> keep;
 };
 
+// One message on the byte transport: `len` bytes at `data`, which either live in
+// `owned` (the sender's bytes were copied, as a socket buffer would hold them) or
+// stay valid for as long as `keep` is held (a sender that hands over a buffer it
+// will not touch again until the exchange is over).
+struct WireMessage {
+    std::vector<uint8_t> owned;
+    const void* data = nullptr;
+    size_t len = 0;
+    std::shared_ptr<void> keep;
+};
+
 class LocalMesh {
 public:
     using Leader = std::function<void(const std::vector<Contribution>&)>;
 
     explicit LocalMesh(int world)
         : world_(world), slots_(static_cast<size_t>(world)),
-          boxes_(static_cast<size_t>(world) * static_cast<size_t>(world)) {}
+          boxes_(static_cast<size_t>(world) * static_cast<size_t>(world)),
+          wires_(static_cast<size_t>(world) * static_cast<size_t>(world)) {}
 
     // Process-wide registry: ranks of one group find their mesh by the key the
     // group's store hands out.
@@ -89,6 +109,15 @@ public:
     void post(int src, int dst, Parcel p);
     Parcel take(int src, int dst, std::chrono::milliseconds timeout);
 
+    // Byte transport (PeerMesh::send / recv, PeerMesh.hpp:19-20).  wire_send never
+    // blocks: the bytes are copied into the message unless `keep` is given, in which
+    // case `buf` is handed over as it is.  wire_recv blocks until the next message
+    // from `src` is there (TimeoutError after `timeout`), requires its length to be
+    // `len` -- the reference's receivers always know how much is coming -- and copies
+    // it into `buf`.
+    void wire_send(int src, int dst, const void* buf, size_t len, std::shared_ptr<void> keep = nullptr);
+    void wire_recv(int src, int dst, void* buf, size_t len, std::chrono::milliseconds timeout);
+
 private:
     const int world_;
     std::mutex mu_;
@@ -102,6 +131,33 @@ private:
     std::mutex box_mu_;
     std::condition_variable box_cv_;
     std::vector<std::deque<Parcel>> boxes_;   // [src * world + dst]
+
+    std::mutex wire_mu_;
+    std::condition_variable wire_cv_;
+    std::vector<std::deque<WireMessage>> wires_;  // [src * world + dst]
+};
+
+// One rank's end of the byte transport, with the reference's PeerMesh interface
+// (csrc/backend/PeerMesh.hpp:12-31): what the reference's algorithms hold as `mesh`.
+class LocalPeer {
+public:
+    LocalPeer(std::shared_ptr<LocalMesh> mesh, int rank, std::chrono::milliseconds timeout)
+        : mesh_(std::move(mesh)), rank_(rank), timeout_(timeout) {}
+
+    void send(int peer, const void* buf, size_t len) { mesh_->wire_send(rank_, peer, buf, len); }
+    void recv(int peer, void* buf, size_t len) { mesh_->wire_recv(peer, rank_, buf, len, timeout_); }
+    // send without the copy: `keep` holds `buf` until the receiver has taken the bytes
+    void send_kept(int peer, const void* buf, size_t len, std::shared_ptr<void> keep) {
+        mesh_->wire_send(rank_, peer, buf, len, std::move(keep));
+    }
+
+    int world() const { return mesh_->world(); }
+    int rank() const { return rank_; }
+
+private:
+    std::shared_ptr<LocalMesh> mesh_;
+    int rank_;
+    std::chrono::milliseconds timeout_;
 };
 
 }  // namespace mccl

@@ -15,6 +15,7 @@
 #include <tuple>
 
 #include "backend/Errors.hpp"
+#include "backend/HostWire.hpp"
 #include "backend/LocalMesh.hpp"
 #include "backend/Logging.hpp"
 #include "backend/Progress.hpp"
@@ -347,6 +348,7 @@ ProcessGroupMCCL::ProcessGroupMCCL(c10::intrusive_ptr<c10d::Store> store, int ra
 
 ProcessGroupMCCL::~ProcessGroupMCCL() {
     if (engine_) engine_->shutdown();
+    host_wire_.reset();
     mesh_.reset();
     shared_.reset();
     if (!mesh_key_.empty()) LocalMesh::forget(mesh_key_);
@@ -358,6 +360,12 @@ std::pair<uint64_t, uint64_t> ProcessGroupMCCL::asyncStats() const {
     return {shared_->async_launches.load(), shared_->async_buckets.load()};
 }
 uint64_t ProcessGroupMCCL::launchCount() const { return ctx_ ? mcclx_launch_count(ctx_) : 0; }
+std::vector<double> ProcessGroupMCCL::wireStats() const {
+    if (!host_wire_) return {};
+    const HostWire::Stats& s = host_wire_->stats();
+    return {static_cast<double>(s.calls), static_cast<double>(s.fold_elems), static_cast<double>(s.fold_peer_bytes),
+            static_cast<double>(s.fold_hbm_bytes), s.fold_ms, static_cast<double>(s.wire_bytes_sent)};
+}
 
 void* ProcessGroupMCCL::my_stream() const {
     return static_cast<void*>(c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(device_)).stream());
@@ -458,13 +466,30 @@ bool env_async_allreduce() {
     const char* e = std::getenv("MCCL_ALLREDUCE_ASYNC");  // re-read on every call, like the other knobs
     return e && e[0] == '1';
 }
+// MCCL_WIRE: unset / "device" = peers' chunks are read where they lie in HBM;
+// "host" = through pinned, device-mapped host memory; "staged" = through the staging pool.
+int env_transport() {
+    const char* e = std::getenv("MCCL_WIRE");
+    if (!e || !*e || std::strcmp(e, "device") == 0) return 0;
+    if (std::strcmp(e, "host") == 0) return 1;
+    if (std::strcmp(e, "staged") == 0) return 2;
+    throw MCCLError(std::string("MCCL_WIRE=") + e + " is not one of device, host, staged");
+}
 }  // namespace
 
 c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tensor>& tensors,
                                                            const c10d::AllreduceOptions& opts) {
     if (getSize() == 1) return make_completed(c10d::OpType::ALLREDUCE, tensors, "mccl:allreduce");
     const int world = getSize();
-    const bool async = env_async_allreduce();
+    int transport = 0;
+    bool async = false;
+    std::string knob_error;
+    try {
+        transport = env_transport();
+        async = transport == 0 && env_async_allreduce();  // the wire modes are synchronous, like the reference
+    } catch (const std::exception& e) {
+        knob_error = e.what();
+    }
     c10::intrusive_ptr<WorkMCCL> work;
     if (async) work = c10::make_intrusive<WorkMCCL>(c10d::OpType::ALLREDUCE, tensors, "mccl:allreduce");
 
@@ -472,6 +497,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
     // message, so that the whole group fails at once instead of waiting for it.
     Contribution c;
     try {
+        if (!knob_error.empty()) throw MCCLError(knob_error);
         MCCL_CHECK(!tensors.empty(), "allreduce: empty tensor list");
         const int op = reduce_op_code(opts.reduceOp);
         const bool wire = env_wire_bf16();
@@ -501,8 +527,38 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
     c.kind = K_ALLREDUCE;
     c.stream = my_stream();
     c.async = async ? 1 : 0;
+    c.transport = transport;
     c.work = work.get();
     flush_engine_();
+
+    if (transport != 0) {
+        // Rank by rank over the byte transport.  The ranks first meet to agree on what
+        // they are about to do (a rank that disagrees, or failed its own checks, fails
+        // everyone at once instead of leaving peers blocked in recv); the meeting also
+        // keeps a fast rank from overwriting its send buffer while a slow one still
+        // reads the previous call's message.
+        const std::vector<uint64_t> numel = c.numel;
+        const std::vector<int> dtype = c.dtype, algo = c.algo;
+        const int op = c.op;
+        const bool wire = c.wire_bf16 != 0;
+        void* stream = c.stream;
+        meet(std::move(c), [world](const std::vector<Contribution>& all) {
+            for (int r = 1; r < world; ++r) {
+                MCCL_CHECK(all[r].transport == all[0].transport, "allreduce: ranks disagree on MCCL_WIRE");
+                MCCL_CHECK(all[r].op == all[0].op && all[r].wire_bf16 == all[0].wire_bf16,
+                           "allreduce: ranks disagree on the reduce op or MCCL_WIRE_DTYPE");
+                MCCL_CHECK(all[r].numel == all[0].numel && all[r].dtype == all[0].dtype,
+                           "allreduce: ranks passed tensors of different size or dtype");
+                MCCL_CHECK(all[r].algo == all[0].algo,
+                           "allreduce: ranks resolved different algorithms (MCCL_ALLREDUCE_ALGO / MCCL_TREE_BELOW differ)");
+            }
+        });
+        if (!host_wire_) host_wire_ = std::make_unique<HostWire>(mesh_, getRank(), device_, opts_.timeout);
+        for (size_t i = 0; i < tensors.size(); ++i)  // one after another (ProcessGroupMCCL.cpp:122-168)
+            host_wire_->allreduce(tensors[i].data_ptr(), dtype[i], numel[i], op, algo[i], wire,
+                                  transport == 1 ? HostWire::Mode::Pinned : HostWire::Mode::Staged, stream);
+        return make_completed(c10d::OpType::ALLREDUCE, tensors, "mccl:allreduce");
+    }
 
     auto shared = shared_;
     const int device = device_;

@@ -30,6 +30,7 @@ namespace mccl {
 
 class Progress;
 class LocalMesh;
+class HostWire;
 struct Contribution;
 
 class ProcessGroupMCCL : public c10d::Backend {
@@ -74,6 +75,9 @@ public:
     // kernel launches the group's reduce queue has issued so far; for tests and the benchmark.
     std::pair<uint64_t, uint64_t> asyncStats() const;
     uint64_t launchCount() const;
+    // The last host-wire allreduce of this rank (MCCL_WIRE=host|staged): elements folded, bytes of
+    // peer operands the fold read, device milliseconds of the fold launch, bytes handed to the wire.
+    std::vector<double> wireStats() const;
 
 private:
     struct Shared;  // reduce queue, scratch and recorded graphs shared by the ranks of one mesh
@@ -92,6 +96,7 @@ private:
     std::shared_ptr<LocalMesh> mesh_;
     std::string mesh_key_;
     std::unique_ptr<Progress> engine_;
+    std::unique_ptr<HostWire> host_wire_;  // MCCL_WIRE=host|staged: this rank's end of the byte transport
     int last_algo_ = -1;
 };
 

@@ -186,6 +186,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         auto* p = dynamic_cast<mccl::ProcessGroupMCCL*>(pg.get());
         return p ? p->asyncStats() : std::pair<uint64_t, uint64_t>(0, 0);
     });
+    m.def("_wire_stats", [](const c10::intrusive_ptr<c10d::Backend>& pg) {
+        auto* p = dynamic_cast<mccl::ProcessGroupMCCL*>(pg.get());
+        return p ? p->wireStats() : std::vector<double>{};
+    });
     m.def("_launch_count", [](const c10::intrusive_ptr<c10d::Backend>& pg) {
         auto* p = dynamic_cast<mccl::ProcessGroupMCCL*>(pg.get());
         return p ? p->launchCount() : uint64_t(0);

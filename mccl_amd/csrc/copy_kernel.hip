@@ -33,34 +33,40 @@ template <> struct Packet<1> { typedef u32x4 type __attribute__((aligned(1))); }
 constexpr int kBlock = 256;
 constexpr int kU = MCCLX_TUNE_COPY_U;
 
+// Up to kFewCopies copies with their descriptors in the kernel arguments:
+// blockIdx.y picks the copy, blockIdx.x one tile of kU * kBlock packets of 16
+// bytes; block 0 of a copy also moves the bytes behind its last whole packet.
+// One tile per block and no loop, like the fold kernels: a uniform 64-bit base
+// plus a 32-bit lane offset per access, and a short path to the first load.
 template <int A>
-__global__ void __launch_bounds__(kBlock) copy_kernel(uint8_t* dst, const uint8_t* src, uint64_t nbytes) {
+__global__ void __launch_bounds__(kBlock) copy_few_kernel(CopyFew a) {
     typedef typename Packet<A>::type V;
-    const MCCLX_GLOBAL uint8_t* gs = (const MCCLX_GLOBAL uint8_t*)src;
-    MCCLX_GLOBAL uint8_t* gd = (MCCLX_GLOBAL uint8_t*)dst;
-    const uint64_t P = nbytes / 16;
-    const uint64_t span = (uint64_t)kU * kBlock;
-    for (uint64_t base = (uint64_t)blockIdx.x * span; base < P; base += (uint64_t)gridDim.x * span) {
-        if (base + span <= P) {
+    const CopyDesc d = a.d[blockIdx.y];
+    const uint64_t P = d.nbytes / 16;
+    const uint64_t first = (uint64_t)blockIdx.x * (kU * kBlock);
+    if (first < P) {
+        const MCCLX_GLOBAL uint8_t* gs = (const MCCLX_GLOBAL uint8_t*)d.src + first * 16;
+        MCCLX_GLOBAL uint8_t* gd = (MCCLX_GLOBAL uint8_t*)d.dst + first * 16;
+        const uint64_t left = P - first;
+        if (left >= (uint64_t)kU * kBlock) {
             u32x4 v[kU];
 #pragma unroll
-            for (int u = 0; u < kU; ++u)
-                v[u] = COPY_LD((const MCCLX_GLOBAL V*)(gs + (base + (uint64_t)u * kBlock + threadIdx.x) * 16));
+            for (int u = 0; u < kU; ++u) v[u] = COPY_LD((const MCCLX_GLOBAL V*)(gs + ((uint32_t)u * kBlock + threadIdx.x) * 16u));
 #pragma unroll
-            for (int u = 0; u < kU; ++u)
-                COPY_ST((MCCLX_GLOBAL V*)(gd + (base + (uint64_t)u * kBlock + threadIdx.x) * 16), v[u]);
+            for (int u = 0; u < kU; ++u) COPY_ST((MCCLX_GLOBAL V*)(gd + ((uint32_t)u * kBlock + threadIdx.x) * 16u), v[u]);
         } else {
-            for (uint64_t p = base + threadIdx.x; p < P; p += kBlock) {
-                u32x4 v = COPY_LD((const MCCLX_GLOBAL V*)(gs + p * 16));
-                COPY_ST((MCCLX_GLOBAL V*)(gd + p * 16), v);
+            for (uint32_t p = threadIdx.x; p < (uint32_t)left; p += kBlock) {
+                u32x4 v = COPY_LD((const MCCLX_GLOBAL V*)(gs + p * 16u));
+                COPY_ST((MCCLX_GLOBAL V*)(gd + p * 16u), v);
             }
         }
     }
     if (blockIdx.x == 0) {
-        uint64_t i = P * 16 + threadIdx.x;
-        if (i < nbytes) gd[i] = gs[i];
+        const uint64_t i = P * 16 + threadIdx.x;
+        if (i < d.nbytes) ((MCCLX_GLOBAL uint8_t*)d.dst)[i] = ((const MCCLX_GLOBAL uint8_t*)d.src)[i];
     }
 }
+
 // One-directional streams with the copy kernel's access shape: what a launch
 // that only reads, or only writes, nbytes costs.  The read keeps its loads alive
 // through a store no input takes (packet XOR == magic, into the buffer's first
@@ -174,23 +180,30 @@ hipError_t launch_stream_probe(hipStream_t st, void* buf, uint64_t nbytes, bool 
     return hipGetLastError();
 }
 
-hipError_t launch_copy(hipStream_t st, void* dst, const void* src, uint64_t nbytes,
-                       uint32_t max_blocks) {
-    if (nbytes == 0) return hipSuccess;
+hipError_t launch_copy_few(hipStream_t st, const CopyFew& a, int align) {
+    uint64_t longest = 0;
+    for (uint32_t i = 0; i < a.n; ++i) longest = a.d[i].nbytes > longest ? a.d[i].nbytes : longest;
+    if (a.n == 0 || longest == 0) return hipSuccess;
     const uint64_t span = (uint64_t)kU * kBlock * 16;
-    uint64_t g = (nbytes + span - 1) / span;
-    if (g > max_blocks) g = max_blocks;
-    if (g < 1) g = 1;
-    uint8_t* d = static_cast<uint8_t*>(dst);
-    const uint8_t* s = static_cast<const uint8_t*>(src);
-    const uintptr_t both = reinterpret_cast<uintptr_t>(d) | reinterpret_cast<uintptr_t>(s);
-    if (both % 4 == 0)
-        copy_kernel<4><<<dim3((uint32_t)g), dim3(kBlock), 0, st>>>(d, s, nbytes);
-    else if (both % 2 == 0)
-        copy_kernel<2><<<dim3((uint32_t)g), dim3(kBlock), 0, st>>>(d, s, nbytes);
+    uint64_t g = (longest + span - 1) / span;
+    if (g >> 31) return hipErrorInvalidValue;
+    const dim3 grid((uint32_t)g, a.n);
+    if (align == 4)
+        copy_few_kernel<4><<<grid, dim3(kBlock), 0, st>>>(a);
+    else if (align == 2)
+        copy_few_kernel<2><<<grid, dim3(kBlock), 0, st>>>(a);
     else
-        copy_kernel<1><<<dim3((uint32_t)g), dim3(kBlock), 0, st>>>(d, s, nbytes);
+        copy_few_kernel<1><<<grid, dim3(kBlock), 0, st>>>(a);
     return hipGetLastError();
+}
+
+hipError_t launch_copy(hipStream_t st, void* dst, const void* src, uint64_t nbytes, uint32_t) {
+    if (nbytes == 0) return hipSuccess;
+    CopyFew a;
+    a.d[0] = CopyDesc{dst, src, nbytes};
+    a.n = 1;
+    const uintptr_t both = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src);
+    return launch_copy_few(st, a, both % 4 == 0 ? 4 : both % 2 == 0 ? 2 : 1);
 }
 
 }  // namespace mcclx

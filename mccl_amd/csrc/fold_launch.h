@@ -94,6 +94,13 @@ struct CopyTable {
     uint32_t uniform_items;  // >0: every copy has this many work items
     uint32_t n;
 };
+// A few copies by value in the kernel arguments (one grid: y = copy, x = tile).
+constexpr int kFewCopies = 32;
+struct CopyFew {
+    CopyDesc d[kFewCopies];
+    uint32_t n;
+};
+hipError_t launch_copy_few(hipStream_t st, const CopyFew& copies, int align);
 // Work items (tiles) one copy of nbytes splits into.
 uint64_t copy_items(uint64_t nbytes);
 // `align`: the widest of 4 / 2 / 1 bytes that every pointer in the table is aligned to.

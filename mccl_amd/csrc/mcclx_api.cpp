@@ -755,12 +755,37 @@ int mcclx_copy_batched(mcclx_ctx* ctx, const mcclx_copy_desc* descs, uint32_t n)
     if (live == 0) return MCCLX_OK;
     DeviceGuard guard(ctx->device);
     if (!guard.ok) return fail(MCCLX_ERR_HIP, "hipSetDevice(%d) failed", ctx->device);
-    // A few large copies: one launch each streams best (a block of the table kernel
-    // first has to fetch its descriptor from memory).  Many small ones: one launch.
-    if (live <= 4 || bytes / live >= (8u << 20)) {
-        for (uint32_t i = 0; i < n; ++i)
-            if (int rc = mcclx_copy(ctx, descs[i].dst, descs[i].src, descs[i].nbytes)) return rc;
-        return MCCLX_OK;
+    const int align = (both % 4 == 0) ? 4 : (both % 2 == 0) ? 2 : 1;
+    // Few or large copies: descriptors in the kernel arguments, up to 32 copies per
+    // grid (a block of the table kernel first has to fetch its descriptor from
+    // memory, which costs large copies 5-10 %); the grid is as wide as the longest
+    // copy of a group, so groups are cut where lengths differ wildly.  Many small
+    // ones: one table launch.
+    if (live <= (uint32_t)mcclx::kFewCopies || bytes / live >= (1u << 20)) {
+        mcclx::CopyFew few;
+        few.n = 0;
+        uint64_t longest = 0, sum = 0;
+        auto flush = [&]() -> int {
+            if (few.n == 0) return MCCLX_OK;
+            hipError_t e = mcclx::launch_copy_few(ctx->stream, few, align);
+            if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "copy_batched launch failed: %s", hipGetErrorString(e));
+            ++ctx->launches;
+            few.n = 0;
+            longest = sum = 0;
+            return MCCLX_OK;
+        };
+        for (uint32_t i = 0; i < n; ++i) {
+            const mcclx_copy_desc& d = descs[i];
+            if (d.nbytes == 0 || d.dst == d.src) continue;
+            const uint64_t lg = d.nbytes > longest ? d.nbytes : longest;
+            // blocks with nothing to do: more than 3 in 4 -> start a new group
+            if (few.n == (uint32_t)mcclx::kFewCopies || (few.n && lg * (few.n + 1) > 4 * (sum + d.nbytes) + (1u << 16)))
+                if (int rc = flush()) return rc;
+            few.d[few.n++] = mcclx::CopyDesc{d.dst, d.src, d.nbytes};
+            longest = d.nbytes > longest ? d.nbytes : longest;
+            sum += d.nbytes;
+        }
+        return flush();
     }
     std::lock_guard<std::mutex> lk(ctx->mu);
     const size_t desc_bytes = (size_t)live * sizeof(mcclx::CopyDesc);
@@ -801,7 +826,6 @@ int mcclx_copy_batched(mcclx_ctx* ctx, const mcclx_copy_desc* descs, uint32_t n)
     t.total_items = (uint32_t)total;
     t.uniform_items = (uint32_t)uniform;
     t.n = live;
-    int align = (both % 4 == 0) ? 4 : (both % 2 == 0) ? 2 : 1;
     hipError_t e = mcclx::launch_copy_many(ctx->stream, t, align, ctx->max_blocks);
     if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "copy_batched launch failed: %s", hipGetErrorString(e));
     ++ctx->launches;

@@ -387,6 +387,86 @@ def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypat
     assert all(all(out[r][2]) for r in range(world)), "a Work was complete when allreduce returned"
 
 
+@pytest.mark.parametrize("transport", ["host", "staged"])
+@pytest.mark.parametrize("algo_name,algo", [("ring", RING), ("butterfly", BUTTERFLY), ("tree", TREE)])
+def test_allreduce_over_the_host_wire_bit_exact(CX, U, monkeypatch, transport, algo_name, algo):
+    """MCCL_WIRE=host|staged: every rank runs its own half of the collective and every chunk
+    crosses the byte transport (send / recv on host memory) -- encoded into pinned memory and
+    read by the owner's fold through the device alias, or staged through the pinned pool.
+    Same bits as the oracle's replay of the reference, for every schedule, op and dtype."""
+    monkeypatch.setenv("MCCL_WIRE", transport)
+    monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", algo_name)
+    monkeypatch.delenv("MCCL_ALLREDUCE_ASYNC", raising=False)
+    rng = np.random.default_rng(70 + algo)
+    cases = [(F32, SUM, 40009, True), (F32, AVG, 70001, True), (F32, SUM, 1237, False), (BF16, AVG, 5003, False),
+             (F16, SUM, 777, False), (F32, MAX, 4099, True), (F32, MIN, 4099, False), (BF16, PRODUCT, 333, False),
+             (F32, SUM, 5, True)]
+    for world in (2, 3, 4):
+        xs = {i: [U.rand_values(rng, n, dt, scale=1e-2, specials=(dt != F16)) for _ in range(world)]
+              for i, (dt, op, n, wire) in enumerate(cases)}
+
+        def fn(r, pg):
+            res = []
+            for i, (dt, op, n, wire) in enumerate(cases):
+                if wire:
+                    os.environ["MCCL_WIRE_DTYPE"] = "bf16"     # every rank sets the same value before the call
+                else:
+                    os.environ.pop("MCCL_WIRE_DTYPE", None)
+                t = U.to_dev(xs[i][r], dt)
+                o = dist.AllreduceOptions(); o.reduceOp = OPS[op]
+                w = pg.allreduce([t], o)
+                assert w.is_completed() and w.wait()
+                res.append(t)
+                pg.barrier().wait()                            # nobody changes the knob while a peer still reads it
+            return res, CX._wire_stats(pg)
+
+        out, errs = run_ranks(CX, world, fn)
+        os.environ.pop("MCCL_WIRE_DTYPE", None)
+        assert errs == [None] * world, errs
+        for i, (dt, op, n, wire) in enumerate(cases):
+            want = [x.copy() for x in xs[i]]
+            rc, used = orc.pg_allreduce(want, dt, op, wire_bf16=wire, env_algo=algo_name)
+            assert rc == 0
+            for r in range(world):
+                if dt == F16:
+                    assert np.array_equal(U.bits(out[r][0][i]), want[r]), (world, i, r)
+                else:
+                    U.assert_same_bits(out[r][0][i], want[r], dt, f"{transport} {algo_name} world {world} case {i} rank {r}")
+        assert all(st[0] == len(cases) for _, st in out)      # every call went over the wire
+
+
+def test_host_wire_error_paths(CX, monkeypatch):
+    monkeypatch.setenv("MCCL_WIRE", "host")
+    world = 2
+
+    def fn(r, pg):
+        msgs = {}
+        try:
+            pg.allreduce([torch.ones(8 + r, device="cuda")])          # sizes differ: found at the meeting point
+        except RuntimeError as e:
+            msgs["mismatch"] = str(e)
+        os.environ["MCCL_WIRE"] = "carrier-pigeon"
+        pg.barrier().wait()
+        try:
+            pg.allreduce([torch.ones(8, device="cuda")])
+        except RuntimeError as e:
+            msgs["knob"] = str(e)
+        pg.barrier().wait()
+        os.environ["MCCL_WIRE"] = "host"
+        pg.barrier().wait()
+        t = torch.full((5,), float(r + 1), device="cuda")
+        pg.allreduce([t]).wait()
+        msgs["after"] = t.cpu().tolist()
+        return msgs
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for m in out:
+        assert "different size or dtype" in m["mismatch"]
+        assert "is not one of device, host, staged" in m["knob"]
+        assert m["after"] == [3.0] * 5
+
+
 def test_reference_collective_vectors(CX):
     """tests/collectives/test_allreduce.py:11-28 (128 x value rank+1, all ops, f32/f16/bf16)
     and tests/test_process_group_local.py:162-207 (3 ranks: SUM = 6, AVG = 2)."""

@@ -129,6 +129,53 @@ def test_c3_ring_110m_ragged_hbm_and_pinned_host(env):
         assert torch.equal(hbm_out[ch].view(torch.int32), fused[0][s:s + c].view(torch.int32))
 
 
+def test_c3_ring_through_the_process_group_with_peers_in_pinned_host_memory(env, monkeypatch):
+    """C3 at full size through the c10d surface: 4 ranks as 4 threads, MCCL_WIRE=host -- every rank
+    encodes what it sends into pinned host memory, the transport delivers into the owner's pinned
+    buffer, and the owner's fold reads its three peers across PCIe.  Same bits as the fused replay
+    with everything in HBM (which the test above checks against the oracle)."""
+    import datetime
+    import threading
+    import torch.distributed as dist
+    from mccl_amd import _C as CX
+    K, H, W, L, U = env
+    world, numel = 4, W.C3["numel"]
+    monkeypatch.setenv("MCCL_WIRE", "host")
+    monkeypatch.setenv("MCCL_WIRE_DTYPE", "bf16")
+    monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "ring")
+    g = torch.Generator(device="cuda").manual_seed(3)
+    base = [torch.randn(numel, device="cuda", generator=g) * 1e-4 for _ in range(world)]
+    want = [t.clone() for t in base]
+    H.allreduce_replay(want, "sum", L.ALGO_RING, wire_bf16=True, mode=FUSED)
+    torch.cuda.synchronize()
+    store = dist.HashStore()
+    stats, errs = [None] * world, [None] * world
+
+    def body(r):
+        try:
+            torch.cuda.set_device(0)
+            pg = CX._create_process_group_mccl(store, r, world, datetime.timedelta(seconds=60))
+            assert pg.allreduce([base[r]]).wait()
+            stats[r] = CX._wire_stats(pg)
+        except BaseException as e:  # noqa: BLE001
+            errs[r] = e
+
+    ts = [threading.Thread(target=body, args=(r,)) for r in range(world)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join(110)
+    assert not any(t.is_alive() for t in ts), "a rank thread hung"
+    assert errs == [None] * world, errs
+    for r in range(world):
+        assert torch.equal(base[r].view(torch.int32), want[r].view(torch.int32)), f"rank {r}"
+    for calls, elems, peer_bytes, hbm_bytes, fold_ms, sent in stats:
+        assert calls == 1 and elems in (27500001, 27499999)
+        assert peer_bytes == 3 * elems * 2 and fold_ms > 0
+        print(f"C3 fold through the backend, peers in pinned host memory: {fold_ms:.2f} ms, "
+              f"{peer_bytes / fold_ms / 1e6:.1f} GB/s over PCIe")
+
+
 def test_c4_tree_4096_messages_one_launch(env):
     K, H, W, L, U = env
     m, n = W.C4["messages"], W.C4["numel"]
