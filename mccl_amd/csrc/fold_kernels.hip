@@ -61,7 +61,29 @@ namespace {
 #define MCCLX_TUNE_PEEL 1   // scalar head peel up to the output's 128-byte boundary
 #endif
 
-constexpr int kBlock = MCCLX_TUNE_BLOCK;  // wavefronts of 64 lanes
+constexpr int kBlock = MCCLX_TUNE_BLOCK;  // threads per block of folds that mix fp32 and 16-bit streams
+#ifndef MCCLX_TUNE_WIDE_BLOCK
+#define MCCLX_TUNE_WIDE_BLOCK 64
+#endif
+#ifndef MCCLX_TUNE_WIDE_U
+#define MCCLX_TUNE_WIDE_U 1
+#endif
+#ifndef MCCLX_TUNE_WIDE_MINK
+#define MCCLX_TUNE_WIDE_MINK 2
+#endif
+#ifndef MCCLX_TUNE_F32_BLOCK
+#define MCCLX_TUNE_F32_BLOCK 64
+#endif
+// Block size by plan, each measured on MI355X.  Folds whose streams all have one
+// element size -- all 16-bit (16 bytes per lane and operand) or all fp32 -- run
+// one-wavefront blocks with one packet per lane: a 512-lane block keeps its wave
+// slots until the last of its loads is back, 64-lane blocks turn them over eight
+// times as often (two to eight 16-bit operands of 512 MiB: +5...9 %, fp32
+// operands: +3...4 %; launches of a few MB are level).  Folds that mix an fp32
+// stream with 16-bit peers (the wire-codec folds) are fastest at 512, and so are
+// one-operand passes.
+constexpr int kWideBlock = MCCLX_TUNE_WIDE_BLOCK;
+constexpr int kWideU = MCCLX_TUNE_WIDE_U;
 
 // Every operand lives in global memory (HBM or host memory mapped into the
 // device).  Pointers that reach a kernel through a descriptor table are
@@ -110,8 +132,20 @@ __device__ __forceinline__ uint32_t bf16_round_bits(float x) {
 
 template <int W> struct Num;  // arithmetic dtype traits
 
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// Besides the scalar rnd (round to W, NaN made canonical where W defines one),
+// every dtype has the array form the packet path uses between the operands of
+// a fold: round_mid rounds E values to W and only guarantees that a NaN stays
+// a NaN -- which NaN is decided once, by canon, after the last operation.  That
+// is the same result as canonicalising after every step (a NaN operand makes a
+// sum or a product NaN whatever its payload; min and max either keep it to the
+// end or drop it), for two instructions per element and step less.
 template <> struct Num<MCCLX_F32> {
     __device__ static __forceinline__ float rnd(float x) { return x; }
+    template <int E> __device__ static __forceinline__ void round_mid(float (&)[E]) {}
+    template <int E> __device__ static __forceinline__ void canon(float (&)[E]) {}
 };
 template <> struct Num<MCCLX_BF16> {
     __device__ static __forceinline__ float rnd(float x) {
@@ -119,6 +153,25 @@ template <> struct Num<MCCLX_BF16> {
     }
     __device__ static __forceinline__ uint32_t enc(float x) { return bf16_round_bits(x) >> 16; }
     __device__ static __forceinline__ float dec(uint32_t h) { return __uint_as_float(h << 16); }
+    // two values per v_cvt_pk_bf16_f32; a NaN whose quiet bit is set (every NaN an
+    // add, a multiply or a decoded bf16 operand can hand over) converts to a NaN
+    template <int E> __device__ static __forceinline__ void round_mid(float (&x)[E]) {
+#if MCCLX_TUNE_HWCVT
+#pragma unroll
+        for (int j = 0; j < E; j += 2) {
+            const uint32_t u = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{x[j], x[j + 1]}, bf16x2));
+            x[j] = __uint_as_float(u << 16);
+            x[j + 1] = __uint_as_float(u & 0xFFFF0000u);
+        }
+#else
+#pragma unroll
+        for (int j = 0; j < E; ++j) x[j] = rnd(x[j]);
+#endif
+    }
+    template <int E> __device__ static __forceinline__ void canon(float (&x)[E]) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) x[j] = (x[j] != x[j]) ? __uint_as_float(0x7FC00000u) : x[j];
+    }
 };
 template <> struct Num<MCCLX_F16> {
     // v_cvt_f16_f32 rounds to nearest even and keeps half denormals.
@@ -130,6 +183,11 @@ template <> struct Num<MCCLX_F16> {
     __device__ static __forceinline__ float dec(uint32_t h) {
         return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
     }
+    template <int E> __device__ static __forceinline__ void round_mid(float (&x)[E]) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) x[j] = rnd(x[j]);
+    }
+    template <int E> __device__ static __forceinline__ void canon(float (&)[E]) {}
 };
 
 // The reference's element operators.  min/max follow the Metal definition
@@ -162,9 +220,13 @@ struct Cfg {
     // no grid-stride looping): one packet per lane streams fastest for folds with
     // an fp32 stream; all-16-bit plans and the one-input codec passes (encode,
     // decode), whose lanes move few bytes, gain 4-12 % from two.
+    static constexpr bool kWide = (E == 8 && K >= MCCLX_TUNE_WIDE_MINK);
     static constexpr int U = MCCLX_TUNE_U ? MCCLX_TUNE_U
+                             : kWide ? kWideU
                              : (TOPO == MCCLX_TOPO_BINOMIAL) ? 1
                              : ((E == 8 || (K == 1 && IO != MCCLX_IO_PURE)) ? 2 : 1);
+    static constexpr int BLOCK = kWide ? kWideBlock
+                                 : (W == MCCLX_F32 && K >= 2) ? MCCLX_TUNE_F32_BLOCK : kBlock;  // threads per block
 };
 
 typedef u32x4 RawPack;  // one packet of one operand: 16 B, or 8 B in .xy (16-bit operand, E = 4)
@@ -221,12 +283,37 @@ __device__ __forceinline__ void load_all(const SegArgs& s, const uint32_t (&pk)[
     if constexpr (k + 1 < C::K) load_all<C, k + 1, U>(s, pk, raw);
 }
 
+// acc = acc (op) v for one packet, rounded to W in STEP mode (NaNs not yet canonical).
+template <class C>
+__device__ __forceinline__ void step_pack(float (&acc)[C::E], const float (&v)[C::E]) {
+#pragma unroll
+    for (int j = 0; j < C::E; ++j) acc[j] = apply<C::OP>(acc[j], v[j]);
+    if constexpr (C::ACC == MCCLX_ACC_STEP) Num<C::W>::template round_mid<C::E>(acc);
+}
+
+// What follows the last operand: the scale, the final rounding of the fp32
+// accumulator mode, and -- if the packet went through any rounding -- the one
+// canonicalisation of NaNs (a fold of one operand without scale moves bits).
+template <class C>
+__device__ __forceinline__ void finish_pack(float (&acc)[C::E], float scale, bool has_scale) {
+    if (has_scale) {
+#pragma unroll
+        for (int j = 0; j < C::E; ++j) acc[j] = acc[j] * scale;
+        if constexpr (C::ACC == MCCLX_ACC_STEP) Num<C::W>::template round_mid<C::E>(acc);
+    }
+    if constexpr (C::ACC != MCCLX_ACC_STEP) Num<C::W>::template round_mid<C::E>(acc);
+    if constexpr (C::K > 1 || C::ACC != MCCLX_ACC_STEP) {
+        Num<C::W>::template canon<C::E>(acc);
+    } else {
+        if (has_scale) Num<C::W>::template canon<C::E>(acc);
+    }
+}
+
 template <class C, int k>
 __device__ __forceinline__ void fold_from(const RawPack (&raw)[C::K], float (&acc)[C::E]) {
     float v[C::E];
     decode<C, k>(raw[k], v);
-#pragma unroll
-    for (int j = 0; j < C::E; ++j) acc[j] = step<C>(acc[j], v[j]);
+    step_pack<C>(acc, v);
     if constexpr (k + 1 < C::K) fold_from<C, k + 1>(raw, acc);
 }
 
@@ -250,9 +337,7 @@ __device__ __forceinline__ void combine(const RawPack (&raw)[C::K], float (&acc)
 #pragma unroll
         for (int mask = 1; mask < C::K; mask <<= 1)
 #pragma unroll
-            for (int r = 0; r + mask < C::K; r += 2 * mask)
-#pragma unroll
-                for (int j = 0; j < C::E; ++j) v[r][j] = step<C>(v[r][j], v[r + mask][j]);
+            for (int r = 0; r + mask < C::K; r += 2 * mask) step_pack<C>(v[r], v[r + mask]);
 #pragma unroll
         for (int j = 0; j < C::E; ++j) acc[j] = v[0][j];
     }
@@ -353,8 +438,7 @@ __device__ __forceinline__ void fold_packs(const SegArgs& s, bool has_out, bool 
         for (int k = 0; k < C::K; ++k) col[k] = raw[k][u];
         float acc[C::E];
         combine<C>(col, acc);
-#pragma unroll
-        for (int j = 0; j < C::E; ++j) acc[j] = finish<C>(acc[j], scale, has_scale);
+        finish_pack<C>(acc, scale, has_scale);
         store_pack<C>(s, has_out, has_wire, pk[u], acc);
     }
 }
@@ -391,7 +475,7 @@ __device__ __forceinline__ SegArgs advanced(const SegArgs& s, uint64_t elems) {
     return t;
 }
 
-// One tile of a segment: after the head peel, the U * kBlock packets from packet
+// One tile of a segment: after the head peel, the U * BLOCK packets from packet
 // `first` on (fewer at the segment's end); the block with `do_edges` also runs
 // the head and the sub-packet tail, one element per lane.  The path to the first
 // load is kept short -- a block lives for about 2 us and eight waves per SIMD
@@ -402,19 +486,20 @@ __device__ __forceinline__ void fold_tile(const SegArgs& s, float scale, bool ha
                                           bool do_edges) {
     constexpr int U = C::U;
     const uint32_t tid = threadIdx.x;
-    const uint32_t head = head_elems<C>(s);  // < 64 <= kBlock
+    constexpr int kB = C::BLOCK;
+    const uint32_t head = head_elems<C>(s);  // < 64 <= kB
     const uint64_t P = (s.count - head) / C::E;
     const bool has_out = s.out != nullptr, has_wire = s.wire_out != nullptr;
     if (first < P) {
         const SegArgs t = advanced<C>(s, head + first * C::E);
         const uint64_t left = P - first;
-        if (left >= (uint64_t)U * kBlock) {
+        if (left >= (uint64_t)U * kB) {
             uint32_t pk[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) pk[u] = (uint32_t)u * kBlock + tid;
+            for (int u = 0; u < U; ++u) pk[u] = (uint32_t)u * kB + tid;
             fold_packs<C, U>(t, has_out, has_wire, pk, scale, has_scale);
         } else {
-            for (uint32_t p = tid; p < (uint32_t)left; p += kBlock) {
+            for (uint32_t p = tid; p < (uint32_t)left; p += kB) {
                 uint32_t one[1] = {p};
                 fold_packs<C, 1>(t, has_out, has_wire, one, scale, has_scale);
             }
@@ -466,7 +551,7 @@ __device__ __forceinline__ void fold_few_body(const FewArgs& a) {
 #if MCCLX_TUNE_TIMELINE
     const uint64_t t_args = wall_clock64();
 #endif
-    const uint64_t span = (uint64_t)C::U * kBlock;
+    const uint64_t span = (uint64_t)C::U * C::BLOCK;
 #if MCCLX_TUNE_XCD
     // workgroups go to the XCDs round robin: block b runs on XCD b % N
     const uint32_t per = grid / MCCLX_TUNE_XCD;  // the grid is a multiple of N
@@ -497,9 +582,9 @@ __device__ __forceinline__ void fold_few_body(const FewArgs& a) {
 template <class C> constexpr bool kLightPlan = C::K <= 4;
 
 template <class C>
-__global__ void __launch_bounds__(kBlock) MCCLX_SGPR_CAP fold_few_kernel(FewArgs a) { fold_few_body<C>(a); }
+__global__ void __launch_bounds__(C::BLOCK) MCCLX_SGPR_CAP fold_few_kernel(FewArgs a) { fold_few_body<C>(a); }
 template <class C>
-__global__ void __launch_bounds__(kBlock) fold_few_wide_kernel(FewArgs a) { fold_few_body<C>(a); }
+__global__ void __launch_bounds__(C::BLOCK) fold_few_wide_kernel(FewArgs a) { fold_few_body<C>(a); }
 
 // A value that is the same in every lane, moved to scalar registers.  The
 // compiler cannot always prove it (a quotient comes out of the vector ALU), and
@@ -521,7 +606,7 @@ __device__ __forceinline__ P* uniptr(P* p) {
 // (checked by the host).
 template <class C>
 __device__ __forceinline__ void fold_table_body(const TableArgs& a) {
-    const uint64_t span = (uint64_t)C::U * kBlock;
+    const uint64_t span = (uint64_t)C::U * C::BLOCK;
     const uint32_t total = (uint32_t)a.total_items;
     const uint32_t uniform = (uint32_t)a.uniform_items;
     for (uint32_t w = blockIdx.x; w < total; w += gridDim.x) {
@@ -558,9 +643,9 @@ __device__ __forceinline__ void fold_table_body(const TableArgs& a) {
 }
 
 template <class C>
-__global__ void __launch_bounds__(kBlock) MCCLX_SGPR_CAP fold_table_kernel(TableArgs a) { fold_table_body<C>(a); }
+__global__ void __launch_bounds__(C::BLOCK) MCCLX_SGPR_CAP fold_table_kernel(TableArgs a) { fold_table_body<C>(a); }
 template <class C>
-__global__ void __launch_bounds__(kBlock) fold_table_wide_kernel(TableArgs a) { fold_table_body<C>(a); }
+__global__ void __launch_bounds__(C::BLOCK) fold_table_wide_kernel(TableArgs a) { fold_table_body<C>(a); }
 
 // ----------------------------------------------------------------- dispatch
 
@@ -592,15 +677,15 @@ static constexpr size_t wide_lds_bytes() { return 0; }
 
 template <class C>
 static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
-    const uint64_t span = (uint64_t)C::U * kBlock * C::E;  // elements per block iteration
+    const uint64_t span = (uint64_t)C::U * C::BLOCK * C::E;  // elements per block iteration
     if (lp.table) {
         TableArgs a = *lp.table;
         uint32_t grid = (uint32_t)(a.total_items < lp.max_blocks ? a.total_items : lp.max_blocks);
         if (grid == 0) return hipSuccess;
         if constexpr (kLightPlan<C>)
-            fold_table_kernel<C><<<dim3(grid), dim3(kBlock), 0, st>>>(a);
+            fold_table_kernel<C><<<dim3(grid), dim3(C::BLOCK), 0, st>>>(a);
         else
-            fold_table_wide_kernel<C><<<dim3(grid), dim3(kBlock), 0, st>>>(a);
+            fold_table_wide_kernel<C><<<dim3(grid), dim3(C::BLOCK), 0, st>>>(a);
     } else {
         FewArgs a = *lp.few;
         uint64_t maxc = 0;
@@ -616,9 +701,9 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
         a.timeline = timeline_next(gx * (uint64_t)a.nseg);
 #endif
         if constexpr (kLightPlan<C>)
-            fold_few_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(kBlock), 0, st>>>(a);
+            fold_few_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(C::BLOCK), 0, st>>>(a);
         else
-            fold_few_wide_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(kBlock), wide_lds_bytes(), st>>>(a);
+            fold_few_wide_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(C::BLOCK), wide_lds_bytes(), st>>>(a);
     }
     return hipGetLastError();
 }
@@ -633,6 +718,7 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
 #define MCCLX_HAS_PART(n) (MCCLX_PART == -1 || MCCLX_PART == (n))
 
 #if MCCLX_HAS_PART(0)
+int plan_block(const PlanKey& key);
 static int key_pack_elems(const PlanKey& key) {
     return (key.dtype == MCCLX_F32 || key.io != MCCLX_IO_PURE) ? 4 : 8;
 }
@@ -641,13 +727,20 @@ uint32_t items_for(const PlanKey& k, uint64_t count) {
     // Mirrors Cfg::U / Cfg::E on the host, for table building.  The head peel
     // only ever removes elements from the packet grid, so this is an upper
     // bound; a tile past the end finds no packets and does nothing.
-    uint64_t span = (uint64_t)plan_unroll(k) * kBlock * key_pack_elems(k);
+    uint64_t span = (uint64_t)plan_unroll(k) * plan_block(k) * key_pack_elems(k);
     uint64_t n = (count + span - 1) / span;
     return (uint32_t)(n ? n : (count ? 1 : 0));
 }
 
+static bool key_is_wide(const PlanKey& key) { return key_pack_elems(key) == 8 && key.k >= MCCLX_TUNE_WIDE_MINK; }
+
+int plan_block(const PlanKey& key) {
+    return key_is_wide(key) ? kWideBlock : (key.dtype == MCCLX_F32 && key.k >= 2 ? MCCLX_TUNE_F32_BLOCK : kBlock);
+}
+
 int plan_unroll(const PlanKey& key) {
     if (MCCLX_TUNE_U) return MCCLX_TUNE_U;
+    if (key_is_wide(key)) return kWideU;
     if (key.topo == MCCLX_TOPO_BINOMIAL) return 1;
     return (key_pack_elems(key) == 8 || (key.k == 1 && key.io != MCCLX_IO_PURE)) ? 2 : 1;
 }
@@ -725,6 +818,10 @@ hipError_t launch_fold(hipStream_t st, const PlanKey& key, const LaunchParams& l
             return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_OUT_F32, 1, 0, 0, 0>>(st, lp);
         if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_PURE && key.k == 2)
             return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_PURE, 2, 0, 0, 0>>(st, lp);
+        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_PURE && key.k == 3)
+            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_PURE, 3, 0, 0, 0>>(st, lp);
+        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_PURE && key.k == 4)
+            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_PURE, 4, 0, 0, 0>>(st, lp);
         if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_PURE && key.k == 1)
             return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_PURE, 1, 0, 0, 0>>(st, lp);
     }

@@ -72,8 +72,9 @@ struct LaunchParams {
     uint32_t max_blocks = 0;           // cap on the grid (persistent sizing)
 };
 
-// Packets-per-lane unroll the kernel template uses for this plan.
+// Packets-per-lane unroll and threads per block the kernel template uses for this plan.
 int plan_unroll(const PlanKey& key);
+int plan_block(const PlanKey& key);
 // Work items (tiles) a segment of `count` elements splits into under this plan.
 uint32_t items_for(const PlanKey& key, uint64_t count);
 // hipErrorInvalidValue = no kernel for this plan.

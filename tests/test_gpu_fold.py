@@ -346,3 +346,55 @@ def test_one_long_segment_among_many_short_ones(K, U):
         K._q(None).fold(K.make_plan(BF16, 2), segs)
         K.hip_sync()
         assert np.array_equal(U.bits(out), want), (nseg, long_n)
+
+
+@pytest.mark.parametrize("k", [2, 3, 5, 8])
+@pytest.mark.parametrize("binomial", [False, True])
+def test_fold_bf16_nan_operands_of_any_payload(K, U, k, binomial):
+    """The packet path rounds between operands without making NaNs canonical and fixes
+    them once at the end.  Pinned here: operands holding every kind of bf16 NaN (quiet and
+    signalling, either sign, payload in any bit), infinities of both signs (whose sum is a
+    NaN born mid-fold) and zeros give what canonicalising after every step gives -- the
+    oracle's result, bit for bit -- for every op, at every operand position."""
+    rng = np.random.default_rng(4000 + k)
+    n = 20011
+    nans = np.array([0x7FC0, 0xFFC0, 0x7F81, 0xFF81, 0x7FFF, 0xFFFF, 0x7FA0, 0x7F80, 0xFF80, 0x0000, 0x8000, 0x3F80],
+                    dtype=np.uint16)
+    for op in (SUM, orc.PRODUCT, orc.MIN, orc.MAX):
+        ins = []
+        for _ in range(k):
+            x = orc.encode_bf16((rng.standard_normal(n)).astype(np.float32))
+            idx = rng.random(n) < 0.15
+            x[idx] = nans[rng.integers(0, nans.size, int(idx.sum()))]
+            ins.append(x)
+        for scale in (None, 1.0 / 3):
+            if scale is not None and op != SUM:
+                continue
+            v = [x.copy() for x in ins]
+            if not binomial:
+                for j in range(1, k):
+                    orc.reduce(v[0], v[j], BF16, op)
+            else:
+                mask = 1
+                while mask < k:
+                    for r in range(0, k - mask, 2 * mask):
+                        orc.reduce(v[r], v[r + mask], BF16, op)
+                    mask <<= 1
+            if scale is not None:
+                orc.scale(v[0], BF16, scale, orc.SCALE_VIEW)
+            d = [U.to_dev(x, BF16) for x in ins]
+            out = torch.empty_like(d[0])
+            plan = K.make_plan(BF16, k, op=op, topo=L().TOPO_BINOMIAL if binomial else L().TOPO_FOLD,
+                               scale_mode=L().SCALE_VIEW if scale else L().SCALE_NONE, scale=scale or 0.0)
+            K._q(None).fold(plan, [K.make_seg(out.data_ptr(), 0, [t.data_ptr() for t in d], n)])
+            K.hip_sync()
+            got = U.bits(out)
+            assert np.array_equal(got, v[0]), f"op {op} k {k} binomial {binomial} scale {scale}: " \
+                f"{int((got != v[0]).sum())} differ, first at {int(np.flatnonzero(got != v[0])[0])}"
+    # one operand, no scale: bits move untouched (a decode keeps a NaN's payload)
+    x = nans.repeat(700)
+    d = U.to_dev(x, BF16)
+    out = torch.empty(x.size, dtype=torch.float32, device="cuda")
+    K._q(None).fold(K.make_plan(BF16, 1, io=L().IO_OUT_F32), [K.make_seg(out.data_ptr(), 0, [d.data_ptr()], x.size)])
+    K.hip_sync()
+    assert np.array_equal(U.bits(out), x.astype(np.uint32) << 16)
