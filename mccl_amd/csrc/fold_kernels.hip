@@ -225,8 +225,9 @@ struct Cfg {
                              : kWide ? kWideU
                              : (TOPO == MCCLX_TOPO_BINOMIAL) ? 1
                              : ((E == 8 || (K == 1 && IO != MCCLX_IO_PURE)) ? 2 : 1);
+    static constexpr bool kDecode = (K == 1 && IO == MCCLX_IO_OUT_F32);  // bf16 -> fp32 cast: +3 % at 64
     static constexpr int BLOCK = kWide ? kWideBlock
-                                 : (W == MCCLX_F32 && K >= 2) ? MCCLX_TUNE_F32_BLOCK : kBlock;  // threads per block
+                                 : ((W == MCCLX_F32 && K >= 2) || kDecode) ? MCCLX_TUNE_F32_BLOCK : kBlock;  // threads per block
 };
 
 typedef u32x4 RawPack;  // one packet of one operand: 16 B, or 8 B in .xy (16-bit operand, E = 4)
@@ -735,7 +736,8 @@ uint32_t items_for(const PlanKey& k, uint64_t count) {
 static bool key_is_wide(const PlanKey& key) { return key_pack_elems(key) == 8 && key.k >= MCCLX_TUNE_WIDE_MINK; }
 
 int plan_block(const PlanKey& key) {
-    return key_is_wide(key) ? kWideBlock : (key.dtype == MCCLX_F32 && key.k >= 2 ? MCCLX_TUNE_F32_BLOCK : kBlock);
+    const bool decode = key.k == 1 && key.io == MCCLX_IO_OUT_F32;
+    return key_is_wide(key) ? kWideBlock : ((key.dtype == MCCLX_F32 && key.k >= 2) || decode ? MCCLX_TUNE_F32_BLOCK : kBlock);
 }
 
 int plan_unroll(const PlanKey& key) {
