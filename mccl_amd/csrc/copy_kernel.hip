@@ -1,7 +1,9 @@
-// copy_kernel.hip -- streaming device copy on the reduce queue: the allgather
+// copy_kernel.hip -- streaming device copies on the reduce queue: the allgather
 // legs (AllreduceAlgos.cpp:77-86, ProcessGroupMCCL.cpp:232-273) and the
-// unstage copy (MPSInterop.mm:408-435).  Also the known-traffic kernel the
-// memory counters are calibrated against.
+// unstage copy (MPSInterop.mm:408-435); a few copies travel by value in the
+// kernel arguments and run as one grid, thousands go through a table.  Also the
+// known-traffic kernel the memory counters are calibrated against, and the
+// read-only / write-only probes a launch's footprint is measured against.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 

@@ -485,9 +485,10 @@ int make_ctx(int device, hipStream_t borrowed, bool borrow, mcclx_ctx** out) {
         return fail(MCCLX_ERR_HIP, "hipGetDeviceProperties failed: %s", hipGetErrorString(e));
     }
     ctx->cus = prop.multiProcessorCount;
-    // Grid cap.  Default: effectively none -- one block per tile measured fastest
-    // (blocks are dispatched in address order; a capped, grid-striding launch
-    // loses 5-20 %).  MCCLX_BLOCKS_PER_CU forces a persistent-style cap.
+    // Grid cap of the table launches.  Default: effectively none -- one block per
+    // tile measured fastest (blocks are dispatched in address order; a capped,
+    // grid-striding launch loses 5-20 %).  MCCLX_BLOCKS_PER_CU forces a
+    // persistent-style cap there; by-value launches always run one block per tile.
     ctx->max_blocks = 1u << 22;
     if (const char* v = getenv("MCCLX_BLOCKS_PER_CU")) {
         int x = atoi(v);
