@@ -81,7 +81,8 @@ HostWire::HostWire(std::shared_ptr<LocalMesh> mesh, int rank, int device, std::c
 
 HostWire::~HostWire() {
     // messages still in flight keep their buffers (and through them the context) alive
-    send_pin_.reset();
+    send_pin_[0].reset();
+    send_pin_[1].reset();
     recv_a_pin_.reset();
     recv_b_pin_.reset();
 }
@@ -143,7 +144,7 @@ void HostWire::allreduce(void* tensor, int dtype, uint64_t numel, int op, int al
         recv_b_dev = device_scratch(recv_b_dev_, send_bytes);
         if (pageable_.size() < max_count * es) pageable_.resize(max_count * es);
     } else {
-        send_keep = pinned(send_pin_, send_bytes);
+        send_keep = pinned(send_pin_[stats_.calls & 1], send_bytes);
         auto a = pinned(recv_a_pin_, recv_a_bytes);
         auto b = pinned(recv_b_pin_, send_bytes);
         send_dev = send_keep->dev;

@@ -75,7 +75,11 @@ private:
     LocalPeer peer_;
     int rank_, world_, device_;
     std::shared_ptr<Ctx> ctx_;
-    std::shared_ptr<Pinned> send_pin_, recv_a_pin_, recv_b_pin_;
+    // Two send buffers, used in turn: a peer may still be copying this rank's last
+    // message of call n out of its send buffer while this rank already encodes call
+    // n+1.  Nobody can finish call n+1 before every rank has finished call n (every
+    // fold needs an operand from every rank), so call n+2 may take call n's buffer.
+    std::shared_ptr<Pinned> send_pin_[2], recv_a_pin_, recv_b_pin_;
     at::Tensor send_dev_, recv_a_dev_, recv_b_dev_;  // Staged mode: the same buffers in HBM
     std::vector<uint8_t> pageable_;                  // Staged mode: where the wire delivers
     Stats stats_;

@@ -75,6 +75,26 @@ def test_mesh_leader_error_reaches_every_rank(CX):
     assert CX._test_mesh(3, 2, -1, 5000, True) == ["[MCCL] leader failed"] * 3
 
 
+# ---- the byte transport with PeerMesh's interface (PeerMesh.hpp:12-31) --------------------
+
+@pytest.mark.parametrize("world", [2, 3, 5])
+def test_peer_send_recv_ring_exchange(CX, world):
+    assert CX._test_peer_wire("ring", world, 8) == ["ok:0"] * world
+
+
+def test_peer_send_kept_hands_the_buffer_over_and_lets_go_of_it(CX):
+    assert CX._test_peer_wire("kept", 3, 8) == ["ok:0"] * 3
+
+
+def test_peer_recv_refuses_a_message_of_another_length(CX):
+    out = CX._test_peer_wire("short", 2)
+    assert all("expects 4 bytes" in o and "which sent 3" in o for o in out), out
+
+
+def test_peer_recv_times_out_and_the_mesh_stays_usable(CX):
+    assert CX._test_peer_wire("silent", 3, 1, 100) == ["timeout:3", "timeout:1", "timeout:2"]
+
+
 # ---- registration: mccl/_backend.py:30-75, tests/test_smoke.py:12-14 ---------------
 
 def test_backend_is_registered_and_registration_is_idempotent():
