@@ -448,6 +448,9 @@ def backend_extras(torch, W):
             out[f"c2_backend_{mode}_us_per_bucket"] = round(max(b for b, _ in res) / nb * 1e6, 1)
             if mode == "async":
                 out["c2_backend_async_launches_for_8_buckets"] = int(res[0][1])
+            # the same with the ranks as native threads: what the interpreter lock shared by
+            # three Python rank threads adds to the figure above
+            out[f"c2_backend_{mode}_native_ranks_us_per_bucket"] = round(max(CX._allreduce_rate(3, numel, nb, 4)), 1)
         os.environ.pop("MCCL_ALLREDUCE_ASYNC", None)
 
         os.environ.update({"MCCL_ALLREDUCE_ALGO": "ring", "MCCL_WIRE": "host"})

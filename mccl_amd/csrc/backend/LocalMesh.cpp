@@ -1,6 +1,7 @@
 #include "backend/LocalMesh.hpp"
 
 #include <atomic>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <unistd.h>
@@ -13,7 +14,19 @@ namespace {
 std::mutex g_registry_mu;
 std::map<std::string, std::weak_ptr<LocalMesh>> g_registry;
 std::atomic<uint64_t> g_next_id{1};
+
+int env_spin_us() {
+    const char* e = std::getenv("MCCL_MEET_SPIN_US");
+    if (!e || !*e) return 200;
+    const long v = std::strtol(e, nullptr, 10);
+    return v < 0 ? 0 : v > 100000 ? 100000 : static_cast<int>(v);
+}
 }  // namespace
+
+LocalMesh::LocalMesh(int world)
+    : world_(world), slots_(static_cast<size_t>(world)), spin_us_(env_spin_us()),
+      boxes_(static_cast<size_t>(world) * static_cast<size_t>(world)),
+      wires_(static_cast<size_t>(world) * static_cast<size_t>(world)) {}
 
 std::string LocalMesh::fresh_key() {
     return "pid" + std::to_string(::getpid()) + "-mesh" + std::to_string(g_next_id.fetch_add(1));
@@ -70,7 +83,13 @@ void LocalMesh::rendezvous(int rank, Contribution c, std::chrono::milliseconds t
         if (err) std::rethrow_exception(err);
         return;
     }
-    auto released = [&] { return generation_ != my_generation || broken_; };
+    auto released = [&] { return generation_.load() != my_generation || broken_.load(); };
+    if (spin_us_ > 0) {
+        lk.unlock();
+        const auto until = std::chrono::steady_clock::now() + std::chrono::microseconds(spin_us_);
+        while (!released() && std::chrono::steady_clock::now() < until) __builtin_ia32_pause();
+        lk.lock();
+    }
     if (timeout.count() <= 0) {
         cv_.wait(lk, released);
     } else if (!cv_.wait_for(lk, timeout, released)) {

@@ -18,6 +18,7 @@
 // the reference's FIFO engine (Progress.hpp:12-18).
 #pragma once
 
+#include <atomic>
 #include <chrono>
 #include <condition_variable>
 #include <cstdint>
@@ -81,10 +82,7 @@ class LocalMesh {
 public:
     using Leader = std::function<void(const std::vector<Contribution>&)>;
 
-    explicit LocalMesh(int world)
-        : world_(world), slots_(static_cast<size_t>(world)),
-          boxes_(static_cast<size_t>(world) * static_cast<size_t>(world)),
-          wires_(static_cast<size_t>(world) * static_cast<size_t>(world)) {}
+    explicit LocalMesh(int world);
 
     // Process-wide registry: ranks of one group find their mesh by the key the
     // group's store hands out.
@@ -99,7 +97,10 @@ public:
     // arrival runs `leader` with every rank's contribution (index = rank);
     // all ranks return when it is done.  If `leader` throws, every rank
     // rethrows that error.  If peers do not arrive within `timeout`, throws
-    // TimeoutError and poisons the mesh (later calls fail at once).
+    // TimeoutError and poisons the mesh (later calls fail at once).  The device work
+    // of a gradient bucket takes tens of microseconds, less than it takes to put a
+    // thread to sleep and wake it: a waiter first polls for MCCL_MEET_SPIN_US
+    // microseconds (default 200, 0 = sleep at once).
     void rendezvous(int rank, Contribution c, std::chrono::milliseconds timeout, const Leader& leader);
 
     // Point-to-point: one FIFO per ordered pair of ranks, as a socket per peer
@@ -124,9 +125,10 @@ private:
     std::condition_variable cv_;
     std::vector<Contribution> slots_;
     int arrived_ = 0;
-    uint64_t generation_ = 0;
+    std::atomic<uint64_t> generation_{0};  // written under mu_; read without it while a waiter spins
     std::exception_ptr last_error_;
-    bool broken_ = false;
+    std::atomic<bool> broken_{false};
+    const int spin_us_;                    // how long a waiter polls before it sleeps (MCCL_MEET_SPIN_US)
 
     std::mutex box_mu_;
     std::condition_variable box_cv_;

@@ -120,11 +120,12 @@ struct ProcessGroupMCCL::Shared {
     bool graphs_enabled = true;
 
     // Event-based completion (MCCL_ALLREDUCE_ASYNC=1).  An allreduce of the group
-    // becomes a Bucket; it is launched at once when the reduce queue is idle and
-    // parked otherwise, and everything parked goes out together -- one launch per
-    // phase for all of it -- as soon as the launch in flight has finished (or a
-    // rank waits on one of the parked Works).  A worker thread waits for each
-    // launch's completion ticket and settles the ranks' Works.
+    // becomes a Bucket.  Up to kDepth launches are kept in flight, so that the queue
+    // always has the next one behind the one that runs; what arrives beyond that is
+    // parked, and everything parked goes out together -- one launch per phase for
+    // all of it -- as soon as a launch in flight has finished (or a rank waits on
+    // one of the parked Works).  A worker thread waits for each launch's completion
+    // ticket, settles the ranks' Works and issues what is parked.
     struct Bucket {
         std::vector<mcclx_replay> reps;
         std::vector<std::vector<void*>> ptrs;  // reps[i].tensors points into ptrs[i]
@@ -132,11 +133,15 @@ struct ProcessGroupMCCL::Shared {
         std::vector<c10::intrusive_ptr<WorkMCCL>> works;  // one per rank
         std::atomic<bool> launched{false};
     };
+    static constexpr uint64_t kDepth = 2;
+    static constexpr size_t kPooledWorkspaces = 16;
     std::mutex amu;
     std::deque<std::shared_ptr<Bucket>> parked;
-    uint64_t inflight_ticket = 0;              // ticket of the newest launch
-    std::atomic<uint64_t> finished_ticket{0};  // newest ticket the completer has seen complete
-    bool flush_scheduled = false;
+    uint64_t launches_issued = 0;                // under amu
+    std::atomic<uint64_t> launches_finished{0};  // counted by the completer, not by polling events: it is
+                                                 // blocked in a wait on the newest event, and a query from
+                                                 // another thread would block with it
+    std::vector<at::Tensor> workspace_pool;      // under amu: workspaces of finished buckets, for reuse
     std::unique_ptr<Progress> completer;
     std::atomic<uint64_t> async_launches{0}, async_buckets{0};
 
@@ -146,8 +151,34 @@ struct ProcessGroupMCCL::Shared {
     }
     ~Shared() {
         if (completer) completer->shutdown();  // settles what is still in flight
+        workspace_pool.clear();
         drop_graphs();
         if (ctx) mcclx_destroy(ctx);
+    }
+
+    // A workspace for one asynchronous call (several may be in flight, each keeps its
+    // own until it has finished).  One that comes back from a finished bucket was last
+    // used on the reduce queue itself and needs no ordering against the allocator.
+    at::Tensor take_workspace(uint64_t nbytes) {
+        {
+            std::lock_guard<std::mutex> lk(amu);
+            size_t best = workspace_pool.size();
+            for (size_t i = 0; i < workspace_pool.size(); ++i) {
+                const auto n = static_cast<uint64_t>(workspace_pool[i].numel());
+                if (n >= nbytes && n <= 2 * nbytes + (1u << 20) &&
+                    (best == workspace_pool.size() || n < static_cast<uint64_t>(workspace_pool[best].numel())))
+                    best = i;
+            }
+            if (best != workspace_pool.size()) {
+                at::Tensor t = std::move(workspace_pool[best]);
+                workspace_pool.erase(workspace_pool.begin() + static_cast<std::ptrdiff_t>(best));
+                return t;
+            }
+        }
+        at::Tensor t = at::empty({static_cast<int64_t>(nbytes)},
+                                 at::TensorOptions().dtype(at::kByte).device(at::kCUDA, device));
+        order_after_allocator(ctx, device);
+        return t;
     }
 
     // Caller holds amu.  Issues the buckets as ONE list replay and hands their
@@ -169,7 +200,7 @@ struct ProcessGroupMCCL::Shared {
                 for (auto& w : b->works) w->finishWithException(err);
             std::rethrow_exception(err);
         }
-        inflight_ticket = ticket;
+        ++launches_issued;
         ++async_launches;
         async_buckets += buckets.size();
         if (!completer) completer = std::make_unique<Progress>();
@@ -181,7 +212,8 @@ struct ProcessGroupMCCL::Shared {
             } catch (...) {
                 failure = std::current_exception();
             }
-            finished_ticket.store(ticket);
+            ++launches_finished;
+            flush_parked();  // first: the queue should not run dry while Works are settled
             for (auto& b : buckets)
                 for (auto& w : b->works) {
                     if (failure)
@@ -189,32 +221,28 @@ struct ProcessGroupMCCL::Shared {
                     else
                         w->finish();
                 }
-            buckets.clear();  // workspaces go back to the allocator only now
+            {
+                std::lock_guard<std::mutex> lk(amu);
+                for (auto& b : buckets)
+                    if (b->workspace.defined() && workspace_pool.size() < kPooledWorkspaces)
+                        workspace_pool.push_back(std::move(b->workspace));
+            }
+            buckets.clear();  // what the pool did not take goes back to the allocator only now
         });
     }
 
-    // Is the newest launch still running?  Answered from what the completer has seen,
-    // not by polling the event: the completer is blocked in a wait on that very event,
-    // and a query from another thread would block with it.
-    bool queue_busy_locked() const { return inflight_ticket != finished_ticket.load(); }
-
     void submit_bucket(std::shared_ptr<Bucket> b) {
         std::lock_guard<std::mutex> lk(amu);
-        if (parked.empty() && !queue_busy_locked()) {
+        // (a launch that finishes after this check takes `amu` after us and finds the bucket parked)
+        if (parked.empty() && launches_issued - launches_finished.load() < kDepth) {
             launch_locked({std::move(b)});
             return;
         }
         parked.push_back(std::move(b));
-        if (!flush_scheduled) {
-            flush_scheduled = true;
-            // runs behind the completion wait of the launch in flight
-            completer->submit([this] { flush_parked(); });
-        }
     }
 
     void flush_parked() {
         std::lock_guard<std::mutex> lk(amu);
-        flush_scheduled = false;
         if (parked.empty()) return;
         std::vector<std::shared_ptr<Bucket>> go(parked.begin(), parked.end());
         parked.clear();
@@ -398,7 +426,7 @@ void ProcessGroupMCCL::meet_built(int kind, void* stream, const std::function<vo
 // allreduce's meeting point while its own engine still owes an earlier
 // collective, or the ranks would meet in different collectives.
 void ProcessGroupMCCL::flush_engine_() {
-    if (!engine_) return;
+    if (!engine_ || engine_->idle()) return;  // only this thread submits: nothing can slip in behind the check
     std::mutex mu;
     std::condition_variable cv;
     bool done = false;
@@ -534,9 +562,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
     if (transport != 0) {
         // Rank by rank over the byte transport.  The ranks first meet to agree on what
         // they are about to do (a rank that disagrees, or failed its own checks, fails
-        // everyone at once instead of leaving peers blocked in recv); the meeting also
-        // keeps a fast rank from overwriting its send buffer while a slow one still
-        // reads the previous call's message.
+        // everyone at once instead of leaving peers blocked in recv).
         const std::vector<uint64_t> numel = c.numel;
         const std::vector<int> dtype = c.dtype, algo = c.algo;
         const int op = c.op;
@@ -571,7 +597,14 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
             MCCL_CHECK(all[r].op == all[0].op && all[r].wire_bf16 == all[0].wire_bf16,
                        "allreduce: ranks disagree on the reduce op or MCCL_WIRE_DTYPE");
             MCCL_CHECK((all[r].async != 0) == async, "allreduce: ranks disagree on MCCL_ALLREDUCE_ASYNC");
-            check_rc(mcclx_queue_wait_stream(ctx, all[r].stream));  // mps_stream_sync, :172
+        }
+        // mps_stream_sync, :172 -- once per distinct stream: ranks on one stream (threads
+        // that all use torch's default stream) are covered by one wait, and a wait costs
+        // the host about ten microseconds
+        for (int r = 0; r < world; ++r) {
+            bool seen = false;
+            for (int q = 0; q < r; ++q) seen = seen || all[q].stream == all[r].stream;
+            if (!seen) check_rc(mcclx_queue_wait_stream(ctx, all[r].stream));
         }
         // one replay per tensor of the list; the reference runs them one after another
         // (ProcessGroupMCCL.cpp:122-168), here a list is issued together so that
@@ -612,9 +645,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
         char* ws = nullptr;
         if (async && total) {
             // several calls may be in flight: each keeps a workspace of its own until it has finished
-            bucket->workspace = at::empty({static_cast<int64_t>(total + 256)},
-                                          at::TensorOptions().dtype(at::kByte).device(at::kCUDA, device));
-            order_after_allocator(ctx, device);
+            bucket->workspace = shared->take_workspace(total + 256);
             auto p = reinterpret_cast<uintptr_t>(bucket->workspace.data_ptr());
             ws = reinterpret_cast<char*>((p + 255) / 256 * 256);
         } else {

@@ -30,6 +30,7 @@ void Progress::submit(Task task) {
         std::lock_guard<std::mutex> lk(mu_);
         if (closing_) return;
         queue_.push_back(std::move(task));
+        ++submitted_;
     }
     wake_.notify_one();
 }
@@ -50,6 +51,11 @@ void Progress::shutdown() {
 size_t Progress::completed() const {
     std::lock_guard<std::mutex> lk(mu_);
     return completed_;
+}
+
+bool Progress::idle() const {
+    std::lock_guard<std::mutex> lk(mu_);
+    return completed_ == submitted_;
 }
 
 void Progress::worker() {

@@ -56,6 +56,8 @@ public:
     void shutdown();
     // Tasks run so far (for tests and diagnostics).
     size_t completed() const;
+    // True when every task submitted so far has run to its end.
+    bool idle() const;
 
 private:
     void worker();
@@ -65,6 +67,7 @@ private:
     std::deque<Task> queue_;
     bool closing_ = false;
     size_t completed_ = 0;
+    size_t submitted_ = 0;
     std::thread thread_;
 };
 

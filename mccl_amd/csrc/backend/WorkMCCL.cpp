@@ -59,6 +59,12 @@ void WorkMCCL::finishWithException(std::exception_ptr error) {
 
 bool WorkMCCL::wait(std::chrono::milliseconds timeout) {
     if (on_wait_) {
+        {
+            // settled already: the device work has been seen to end, nothing to order against
+            std::lock_guard<std::mutex> lk(mu_);
+            if (state_ == State::Succeeded) return true;
+            if (state_ == State::Failed) std::rethrow_exception(error_);
+        }
         on_wait_();  // stream-ordered: the caller's stream now waits for the result on the device
         std::lock_guard<std::mutex> lk(mu_);
         if (state_ == State::Failed) std::rethrow_exception(error_);

@@ -34,8 +34,9 @@ public:
     // Event-based completion: with a wait hook, wait() does not block the host until
     // the Work is settled.  It runs the hook -- which makes the caller's stream wait,
     // on the device, for the reduce queue -- and returns; the Work and its Future
-    // settle later, when the device has finished.  A Work that has already failed
-    // still rethrows from wait().
+    // settle later, when the device has finished.  A Work that has settled by the
+    // time of the wait needs no hook (the device work is known to be over); one that
+    // has failed rethrows from wait().
     void setWaitHook(std::function<void()> on_wait) { on_wait_ = std::move(on_wait); }
     void finish();
     void finishWithException(std::exception_ptr error);

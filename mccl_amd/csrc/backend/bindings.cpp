@@ -10,7 +10,10 @@
 #include <pybind11/functional.h>
 #include <pybind11/stl.h>
 
+#include <c10/hip/HIPFunctions.h>
+#include <c10/hip/HIPStream.h>
 #include <torch/csrc/distributed/c10d/Backend.hpp>
+#include <torch/csrc/distributed/c10d/HashStore.hpp>
 #include <torch/csrc/distributed/c10d/Store.hpp>
 
 #include <atomic>
@@ -154,6 +157,127 @@ std::vector<std::string> mesh_probe(int world, int rounds, int absent, int timeo
     return out;
 }
 
+// `world` ranks as native threads, each with its own process group on device 0,
+// issue `buckets` allreduces of `numel` floats back to back and wait for them;
+// the best of `rounds` rounds, in microseconds per bucket, for every rank.  What
+// the c10d surface costs without an interpreter in the ranks' way (the knobs are
+// read from the environment as always).
+std::vector<double> allreduce_rate_probe(int world, int64_t numel, int buckets, int rounds) {
+    auto store = c10::make_intrusive<c10d::HashStore>();
+    std::vector<double> best(static_cast<size_t>(world), 1e30);
+    std::vector<std::string> errs(static_cast<size_t>(world));
+    std::vector<std::thread> ts;
+    for (int r = 0; r < world; ++r)
+        ts.emplace_back([&, r] {
+            try {
+                c10::hip::set_device(0);
+                mccl::ProcessGroupMCCL::Options opts;
+                opts.timeout = std::chrono::milliseconds(120000);
+                auto pg = c10::make_intrusive<mccl::ProcessGroupMCCL>(store, r, world, opts);
+                std::vector<std::vector<at::Tensor>> lists;
+                for (int b = 0; b < buckets; ++b)
+                    lists.push_back({at::randn({numel}, at::TensorOptions().device(at::kCUDA, 0)) * 1e-3});
+                c10d::AllreduceOptions o;
+                o.reduceOp = c10d::ReduceOp::AVG;
+                auto stream = c10::hip::getCurrentHIPStream(0);
+                for (int rep = 0; rep < rounds; ++rep) {
+                    stream.synchronize();
+                    pg->barrier()->wait();
+                    const auto t0 = std::chrono::steady_clock::now();
+                    std::vector<c10::intrusive_ptr<c10d::Work>> works;
+                    for (auto& l : lists) works.push_back(pg->allreduce(l, o));
+                    for (auto& w : works) w->wait();
+                    stream.synchronize();
+                    const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+                    best[static_cast<size_t>(r)] = std::min(best[static_cast<size_t>(r)], us / buckets);
+                }
+                stream.synchronize();
+                pg->barrier()->wait();
+            } catch (const std::exception& e) {
+                errs[static_cast<size_t>(r)] = e.what();
+            }
+        });
+    for (auto& t : ts) t.join();
+    for (auto& e : errs)
+        if (!e.empty()) throw mccl::MCCLError(e);
+    return best;
+}
+
+// The byte transport with PeerMesh's interface, between `world` threads.
+//  "ring":    `rounds` ring steps as the reference's allreduce_ring issues them (send to
+//             the right neighbour, receive from the left; AllreduceAlgos.cpp:62-69) with
+//             messages of growing length; every rank checks what it received byte by byte.
+//  "kept":    the same with send_kept: the payload is not copied, and the receiver's copy
+//             must release the sender's hold on the buffer.
+//  "short":   the receiver expects more bytes than were sent.
+//  "silent":  nobody sends; recv must time out and leave the mesh usable for a later exchange.
+std::vector<std::string> peer_wire_probe(const std::string& mode, int world, int rounds, int timeout_ms) {
+    auto mesh = mccl::LocalMesh::create(mccl::LocalMesh::fresh_key(), world);
+    std::vector<std::string> out(static_cast<size_t>(world));
+    std::vector<std::thread> ts;
+    auto pattern = [](int from, int round, size_t i) { return static_cast<uint8_t>(from * 31 + round * 7 + i * 13 + 1); };
+    for (int r = 0; r < world; ++r)
+        ts.emplace_back([&, r] {
+            mccl::LocalPeer peer(mesh, r, std::chrono::milliseconds(timeout_ms));
+            const int right = (r + 1) % world, left = (r + world - 1) % world;
+            try {
+                if (mode == "silent") {
+                    std::string first;
+                    uint8_t b = 0;
+                    try {
+                        peer.recv(left, &b, 1);
+                        first = "received";
+                    } catch (const mccl::TimeoutError& e) {
+                        first = "timeout";
+                    }
+                    // nobody sends before everybody has seen the silence
+                    mesh->rendezvous(r, mccl::Contribution{}, std::chrono::milliseconds(20000),
+                                     [](const std::vector<mccl::Contribution>&) {});
+                    uint8_t mine = static_cast<uint8_t>(r + 1), theirs = 0;
+                    mccl::LocalPeer patient(mesh, r, std::chrono::milliseconds(20000));
+                    patient.send(right, &mine, 1);
+                    patient.recv(left, &theirs, 1);
+                    out[static_cast<size_t>(r)] = first + ":" + std::to_string(theirs);
+                    return;
+                }
+                if (mode == "short") {
+                    uint8_t three[3] = {1, 2, 3}, four[4] = {0, 0, 0, 0};
+                    peer.send(right, three, 3);
+                    peer.recv(left, four, 4);
+                    out[static_cast<size_t>(r)] = "accepted";
+                    return;
+                }
+                long held = 0;
+                std::shared_ptr<std::vector<uint8_t>> previous;
+                for (int i = 0; i < rounds; ++i) {
+                    const size_t len = static_cast<size_t>(i) * 1000 + (i == 0 ? 0 : 17);  // round 0: an empty message
+                    auto buf = std::make_shared<std::vector<uint8_t>>(len);
+                    for (size_t k = 0; k < len; ++k) (*buf)[k] = pattern(r, i, k);
+                    if (mode == "kept")
+                        peer.send_kept(right, buf->data(), len, buf);
+                    else
+                        peer.send(right, buf->data(), len);
+                    if (mode != "kept") std::fill(buf->begin(), buf->end(), 0);  // a copy was taken: ours to reuse
+                    std::vector<uint8_t> got(len, 0xEE);
+                    peer.recv(left, got.data(), len);
+                    for (size_t k = 0; k < len; ++k)
+                        if (got[k] != pattern(left, i, k)) throw mccl::MCCLError("wrong byte in round " + std::to_string(i));
+                    if (mode == "kept") {
+                        // our message is released once the right neighbour has taken it; it
+                        // takes it before it can send us round i+1, so check one round late
+                        if (previous && previous.use_count() != 1) ++held;
+                        previous = buf;
+                    }
+                }
+                out[static_cast<size_t>(r)] = "ok:" + std::to_string(held);
+            } catch (const std::exception& e) {
+                out[static_cast<size_t>(r)] = e.what();
+            }
+        });
+    for (auto& t : ts) t.join();
+    return out;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -206,6 +330,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::call_guard<py::gil_scoped_release>());
     m.def("_test_work", &work_probe, py::arg("mode"), py::arg("wait_ms") = 1000,
           py::call_guard<py::gil_scoped_release>());
+    m.def("_allreduce_rate", &allreduce_rate_probe, py::arg("world"), py::arg("numel"), py::arg("buckets") = 8,
+          py::arg("rounds") = 4, py::call_guard<py::gil_scoped_release>(),
+          "Microseconds per allreduce, per rank, with the ranks as native threads of this process.");
+    m.def("_test_peer_wire", &peer_wire_probe, py::arg("mode"), py::arg("world") = 3, py::arg("rounds") = 6,
+          py::arg("timeout_ms") = 5000, py::call_guard<py::gil_scoped_release>());
     m.def("_test_mesh", &mesh_probe, py::arg("world"), py::arg("rounds") = 3, py::arg("absent") = -1,
           py::arg("timeout_ms") = 2000, py::arg("leader_throws") = false,
           py::call_guard<py::gil_scoped_release>());

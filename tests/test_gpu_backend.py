@@ -335,13 +335,13 @@ def test_divergent_argument_error_fails_every_rank_at_once(CX):
 def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypatch):
     """MCCL_ALLREDUCE_ASYNC=1: allreduce returns a pending Work, wait() orders the caller's
     stream after the reduce queue without blocking the host, the Future settles from the
-    completion ticket, and buckets issued while an earlier one is still running go out
-    together (one launch per phase for all of them).  Results are the oracle's, bit for bit."""
+    completion ticket, and buckets issued while two earlier launches are still in flight go
+    out together (one launch per phase for all of them).  Results are the oracle's, bit for bit."""
     monkeypatch.setenv("MCCL_ALLREDUCE_ASYNC", "1")
     monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "butterfly")
     monkeypatch.setenv("MCCL_WIRE_DTYPE", "bf16")
     world = 3
-    sizes = [6_553_600, 1_000_003, 70_001, 1_000_003]
+    sizes = [6_553_600, 1_000_003, 70_001, 1_000_003, 33]
     rng = np.random.default_rng(31)
     xs = [[(rng.standard_normal(n) * 1e-3).astype(np.float32) for _ in range(world)] for n in sizes]
 
@@ -382,8 +382,8 @@ def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypat
     (l0, b0), k0 = out[0][3]
     (l1, b1), k1 = out[0][4]
     assert b1 - b0 == len(sizes)
-    assert l1 - l0 == 2, "the first bucket alone, the three behind it together"
-    assert k1 - k0 == 3 * 2, "a launch of several buckets is encode + fold + cast, once"
+    assert l1 - l0 == 3, "two buckets go out at once to keep the queue fed, the three behind them together"
+    assert k1 - k0 == 3 * 3, "a launch of several buckets is encode + fold + cast, once"
     assert all(all(out[r][2]) for r in range(world)), "a Work was complete when allreduce returned"
 
 
@@ -433,6 +433,37 @@ def test_allreduce_over_the_host_wire_bit_exact(CX, U, monkeypatch, transport, a
                 else:
                     U.assert_same_bits(out[r][0][i], want[r], dt, f"{transport} {algo_name} world {world} case {i} rank {r}")
         assert all(st[0] == len(cases) for _, st in out)      # every call went over the wire
+
+
+@pytest.mark.parametrize("transport", ["host", "staged"])
+def test_host_wire_tensor_list_of_unequal_sizes(CX, U, monkeypatch, transport):
+    """A list goes over the wire one tensor after another with no meeting in between
+    (ProcessGroupMCCL.cpp:122-168): a rank may start on the next tensor while a peer still
+    takes delivery of the last one, and consecutive tensors lay their chunks out differently."""
+    monkeypatch.setenv("MCCL_WIRE", transport)
+    monkeypatch.setenv("MCCL_WIRE_DTYPE", "bf16")
+    monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "ring")
+    rng = np.random.default_rng(91)
+    world, sizes = 3, [300007, 11, 65536, 3, 200001, 4097]
+    for op in (SUM, MAX):
+        xs = [[U.rand_values(rng, n, F32, scale=1e-2) for n in sizes] for _ in range(world)]
+
+        def fn(r, pg):
+            ts = [U.to_dev(x, F32) for x in xs[r]]
+            o = dist.AllreduceOptions(); o.reduceOp = OPS[op]
+            for _ in range(3):                      # the same buffers again: results are idempotent only for MAX
+                pg.allreduce([t.clone() for t in ts], o).wait()
+            pg.allreduce(ts, o).wait()
+            return ts
+
+        out, errs = run_ranks(CX, world, fn)
+        assert errs == [None] * world, errs
+        for i, n in enumerate(sizes):
+            want = [xs[r][i].copy() for r in range(world)]
+            rc, _ = orc.pg_allreduce(want, F32, op, wire_bf16=True, env_algo="ring")
+            assert rc == 0
+            for r in range(world):
+                U.assert_same_bits(out[r][i], want[r], F32, f"{transport} op {op} tensor {i} rank {r}")
 
 
 def test_host_wire_error_paths(CX, monkeypatch):
