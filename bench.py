@@ -247,14 +247,28 @@ def main():
 
 
 def cpu_model() -> str:
+    """The host CPU as /proc/cpuinfo names it; a virtualised box may only say "AMD EPYC",
+    so the family / model numbers and the clock go with it."""
+    want = {"model name": None, "cpu family": None, "model": None, "cpu mhz": None}
     try:
         with open("/proc/cpuinfo") as f:
             for line in f:
-                if line.lower().startswith("model name"):
-                    return line.split(":", 1)[1].strip()
+                key, _, val = line.partition(":")
+                key = key.strip().lower()
+                if key in want and want[key] is None:
+                    want[key] = val.strip()
+                if all(v is not None for v in want.values()):
+                    break
     except OSError:
         pass
-    return "unknown"
+    if want["model name"] is None:
+        return "unknown"
+    extra = []
+    if want["cpu family"] and want["model"]:
+        extra.append(f"family {want['cpu family']} model {want['model']}")
+    if want["cpu mhz"]:
+        extra.append(f"{float(want['cpu mhz']):.0f} MHz")
+    return want["model name"] + (f" ({', '.join(extra)})" if extra else "")
 
 
 def timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure, bytes_per_step):
