@@ -31,7 +31,9 @@ extern "C" {
 #endif
 
 #define MCCLX_API __attribute__((visibility("default")))
-#define MCCLX_ABI_VERSION 1
+/* 2: mcclx_plan.flags (was a reserved field that had to be 0), mcclx_fold_batched_noalloc,
+ *    mcclx_probe_stream.  Layouts of version 1 callers stay valid. */
+#define MCCLX_ABI_VERSION 2
 #define MCCLX_MAX_INPUTS 8 /* inputs one launch folds; wider worlds chain launches */
 
 /* ---- codes ---------------------------------------------------------------- */
@@ -173,7 +175,7 @@ typedef struct {
  * and, for the *_F32 io modes, its encode/decode casts). */
 MCCLX_API int mcclx_fold(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* seg);
 
-/* One persistent-block launch over `nseg` independent segments sharing a plan:
+/* One launch over `nseg` independent segments sharing a plan:
  * the tree path's many sub-256 KB messages, or all virtual ranks' chunks of
  * one schedule phase.  Segment descriptors are copied before the call returns. */
 MCCLX_API int mcclx_fold_batched(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs,

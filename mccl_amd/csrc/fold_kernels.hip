@@ -144,6 +144,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 // end or drop it), for two instructions per element and step less.
 template <> struct Num<MCCLX_F32> {
     __device__ static __forceinline__ float rnd(float x) { return x; }
+    __device__ static __forceinline__ float scaled(float x, float s) { return x * s; }
     template <int E> __device__ static __forceinline__ void round_mid(float (&)[E]) {}
     template <int E> __device__ static __forceinline__ void canon(float (&)[E]) {}
 };
@@ -153,6 +154,7 @@ template <> struct Num<MCCLX_BF16> {
     }
     __device__ static __forceinline__ uint32_t enc(float x) { return bf16_round_bits(x) >> 16; }
     __device__ static __forceinline__ float dec(uint32_t h) { return __uint_as_float(h << 16); }
+    __device__ static __forceinline__ float scaled(float x, float s) { return x * s; }
     // two values per v_cvt_pk_bf16_f32; a NaN whose quiet bit is set (every NaN an
     // add, a multiply or a decoded bf16 operand can hand over) converts to a NaN
     template <int E> __device__ static __forceinline__ void round_mid(float (&x)[E]) {
@@ -182,6 +184,13 @@ template <> struct Num<MCCLX_F16> {
     }
     __device__ static __forceinline__ float dec(uint32_t h) {
         return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+    }
+    // x and the scale constant are both half values, so the half product IS the rounded
+    // fp32 product (two 11-bit significands multiply exactly in fp32).  Written as a half
+    // multiply on purpose: "round(x * s)" in fp32 is selected as a mixed-precision
+    // fma(s, x, +0), which turns a product of -0 into +0.
+    __device__ static __forceinline__ float scaled(float x, float s) {
+        return (float)((_Float16)x * (_Float16)s);
     }
     template <int E> __device__ static __forceinline__ void round_mid(float (&x)[E]) {
 #pragma unroll
@@ -269,7 +278,7 @@ __device__ __forceinline__ float step(float a, float b) {
 template <class C>
 __device__ __forceinline__ float finish(float acc, float scale, bool has_scale) {
     if (has_scale) {
-        acc = acc * scale;
+        acc = Num<C::W>::scaled(acc, scale);
         if constexpr (C::ACC == MCCLX_ACC_STEP) acc = Num<C::W>::rnd(acc);
     }
     if constexpr (C::ACC != MCCLX_ACC_STEP) acc = Num<C::W>::rnd(acc);
@@ -299,7 +308,7 @@ template <class C>
 __device__ __forceinline__ void finish_pack(float (&acc)[C::E], float scale, bool has_scale) {
     if (has_scale) {
 #pragma unroll
-        for (int j = 0; j < C::E; ++j) acc[j] = acc[j] * scale;
+        for (int j = 0; j < C::E; ++j) acc[j] = Num<C::W>::scaled(acc[j], scale);
         if constexpr (C::ACC == MCCLX_ACC_STEP) Num<C::W>::template round_mid<C::E>(acc);
     }
     if constexpr (C::ACC != MCCLX_ACC_STEP) Num<C::W>::template round_mid<C::E>(acc);

@@ -398,3 +398,37 @@ def test_fold_bf16_nan_operands_of_any_payload(K, U, k, binomial):
     K._q(None).fold(K.make_plan(BF16, 1, io=L().IO_OUT_F32), [K.make_seg(out.data_ptr(), 0, [d.data_ptr()], x.size)])
     K.hip_sync()
     assert np.array_equal(U.bits(out), x.astype(np.uint32) << 16)
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
+@pytest.mark.parametrize("op", [SUM, orc.PRODUCT])
+def test_scale_after_a_fold_keeps_the_sign_of_zero(K, U, dtype, op):
+    """-0 * (1/N) is -0.  Sums of negative zeros and products that underflow produce
+    negative zeros in bulk; the scale that follows (the AVG of AllreduceAlgos.cpp:88-91,
+    the fused accumulate_scale kernels, shaders.metal:447-551) must hand them on."""
+    rng = np.random.default_rng(77 + dtype + op)
+    n = 20011
+    for k in (1, 2, 3, 6):
+        ins = [U.rand_values(rng, n, dtype, scale=1e-3) for _ in range(k)]
+        zeros = rng.choice(n, size=n // 4, replace=False)
+        for x in ins:                                  # a quarter of the elements: zeros of either sign
+            sign = rng.random(zeros.size) < 0.8
+            if dtype == F32:
+                x[zeros] = np.where(sign, np.float32(-0.0), np.float32(0.0))
+            else:
+                x[zeros] = np.where(sign, np.uint16(0x8000), np.uint16(0))
+        for scale, mode_o, mode_x in ((0.5, orc.SCALE_VIEW, L().SCALE_VIEW), (1.0 / 3, orc.SCALE_TENSOR, L().SCALE_TENSOR)):
+            v = [x.copy() for x in ins]
+            for j in range(1, k):
+                orc.reduce(v[0], v[j], dtype, op)
+            orc.scale(v[0], dtype, scale, mode_o)
+            assert (U.np_bits(v[0]) == (0x80000000 if dtype == F32 else 0x8000)).sum() > n // 100, "the case needs -0 results"
+            d = [U.to_dev(x, dtype) for x in ins]
+            out = torch.empty_like(d[0])
+            plan = K.make_plan(dtype, k, op=op, scale_mode=mode_x, scale=scale)
+            K._q(None).fold(plan, [K.make_seg(out.data_ptr(), 0, [t.data_ptr() for t in d], n)])
+            K.hip_sync()
+            if dtype == F16:
+                assert np.array_equal(U.bits(out), v[0]), (op, k, scale)
+            else:
+                U.assert_same_bits(out, v[0], dtype, f"dtype {dtype} op {op} k {k} scale {scale}")
