@@ -332,16 +332,20 @@ def test_divergent_argument_error_fails_every_rank_at_once(CX):
         assert ok == [6.0] * 5
 
 
-def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypatch):
+@pytest.mark.parametrize("queues", [1, 2])
+def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypatch, queues):
     """MCCL_ALLREDUCE_ASYNC=1: allreduce returns a pending Work, wait() orders the caller's
     stream after the reduce queue without blocking the host, the Future settles from the
     completion ticket, and buckets issued while two earlier launches are still in flight go
-    out together (one launch per phase for all of them).  Results are the oracle's, bit for bit."""
+    out together (one launch per phase for all of them).  With two queues (the default) the
+    buckets alternate between them, up to two launches in flight on each.  Results are the oracle's,
+    bit for bit."""
     monkeypatch.setenv("MCCL_ALLREDUCE_ASYNC", "1")
+    monkeypatch.setenv("MCCL_ASYNC_QUEUES", str(queues))
     monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "butterfly")
     monkeypatch.setenv("MCCL_WIRE_DTYPE", "bf16")
     world = 3
-    sizes = [6_553_600, 1_000_003, 70_001, 1_000_003, 33]
+    sizes = [6_553_600, 1_000_003, 70_001, 1_000_003, 33, 4097, 250_000]
     rng = np.random.default_rng(31)
     xs = [[(rng.standard_normal(n) * 1e-3).astype(np.float32) for _ in range(world)] for n in sizes]
 
@@ -382,9 +386,65 @@ def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypat
     (l0, b0), k0 = out[0][3]
     (l1, b1), k1 = out[0][4]
     assert b1 - b0 == len(sizes)
-    assert l1 - l0 == 3, "two buckets go out at once to keep the queue fed, the three behind them together"
-    assert k1 - k0 == 3 * 3, "a launch of several buckets is encode + fold + cast, once"
+    if queues == 1:
+        assert l1 - l0 == 3, "two buckets go out at once to keep the queue fed, the five behind them together"
+    else:
+        assert l1 - l0 == 6, "two buckets at once on either queue; behind them buckets 4 and 6 together, and bucket 5"
+    assert k1 - k0 == 3 * (l1 - l0), "a launch of several buckets is encode + fold + cast, once"
     assert all(all(out[r][2]) for r in range(world)), "a Work was complete when allreduce returned"
+
+
+@pytest.mark.parametrize("queues", [1, 2])
+def test_event_based_allreduces_that_share_memory_run_in_program_order(CX, U, monkeypatch, queues):
+    """Event-based launches alternate between two queues and may overlap on the device; calls
+    that touch the same tensor must still take effect one after another, also across other
+    collectives issued in between, with nobody waiting on a Work until the end."""
+    monkeypatch.setenv("MCCL_ALLREDUCE_ASYNC", "1")
+    monkeypatch.setenv("MCCL_ASYNC_QUEUES", str(queues))
+    monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "ring")
+    monkeypatch.delenv("MCCL_WIRE_DTYPE", raising=False)
+    world, n = 3, 700_001
+    rng = np.random.default_rng(5)
+    a = [(rng.standard_normal(n) * 1e-2).astype(np.float32) for _ in range(world)]
+    b = [(rng.standard_normal(n) * 1e-2).astype(np.float32) for _ in range(world)]
+
+    def fn(r, pg):
+        ta, tb = U.to_dev(a[r], F32), U.to_dev(b[r], F32)
+        gathered = torch.empty(world * n, dtype=torch.float32, device="cuda")
+        big = torch.empty(1 << 28, dtype=torch.uint8, device="cuda") if r == 0 else None
+        torch.cuda.current_stream().synchronize()
+        if r == 0:                                   # keep the queues busy, so that launches pile up
+            for _ in range(20):
+                big[: 1 << 27].copy_(big[1 << 27:])
+        works = []
+        smax = dist.AllreduceOptions(); smax.reduceOp = dist.ReduceOp.MAX
+        works.append(pg.allreduce([ta]))             # a = sum(a)
+        works.append(pg.allreduce([tb], smax))       # b = max(b)                 (other queue, independent)
+        works.append(pg.allreduce([ta]))             # a = 3 * sum(a)             (other queue than the first)
+        works.append(pg.allreduce([ta, tb]))         # a = 9 * sum(a), b = 3 * max(b)
+        bo = dist.BroadcastOptions(); bo.rootRank = 1
+        works.append(pg.broadcast([tb], bo))         # on the main queue, behind all of the above
+        works.append(pg.allreduce([tb]))             # b = 3 * (3 * max(b))
+        works.append(pg._allgather_base(gathered, ta))
+        for w in works:
+            w.wait()
+        torch.cuda.current_stream().synchronize()
+        return ta, tb, gathered
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    wa = [x.copy() for x in a]
+    wb = [x.copy() for x in b]
+    for _ in range(3):
+        assert orc.pg_allreduce(wa, F32, SUM, env_algo="ring")[0] == 0
+    assert orc.pg_allreduce(wb, F32, MAX, env_algo="ring")[0] == 0
+    assert orc.pg_allreduce(wb, F32, SUM, env_algo="ring")[0] == 0
+    wb = [wb[1].copy() for _ in range(world)]
+    assert orc.pg_allreduce(wb, F32, SUM, env_algo="ring")[0] == 0
+    for r in range(world):
+        U.assert_same_bits(out[r][0], wa[r], F32, f"a on rank {r}")
+        U.assert_same_bits(out[r][1], wb[r], F32, f"b on rank {r}")
+        U.assert_same_bits(out[r][2], np.concatenate(wa), F32, f"gathered on rank {r}")
 
 
 @pytest.mark.parametrize("transport", ["host", "staged"])
