@@ -75,7 +75,9 @@ enum {
 
 enum {
     MCCLX_ACC_STEP = 0, /* round to W after every operation: bit-exact to the reference   */
-    MCCLX_ACC_F32 = 1   /* NOT the reference: fp32 accumulator, one final rounding         */
+    MCCLX_ACC_F32 = 1   /* NOT the reference: fp32 accumulator, the scale applied as
+                           (float)scale in fp32, one final rounding (inside one fold: a
+                           world wider than MCCLX_MAX_INPUTS chains folds and rounds between) */
 };
 
 enum { MCCLX_ALGO_RING = 0, MCCLX_ALGO_TREE = 1, MCCLX_ALGO_BUTTERFLY = 2 };

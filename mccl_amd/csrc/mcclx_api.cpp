@@ -229,8 +229,11 @@ int check_plan(const mcclx_plan* p, mcclx::PlanKey* key, float* scale_f, int* ha
     *key = mcclx::PlanKey{p->dtype, p->io, p->k, (p->k >= 4) ? p->topo : MCCLX_TOPO_FOLD, op, acc};
     *has_scale = p->scale_mode != MCCLX_SCALE_NONE;
     *scale_f = 1.0f;
-    if (*has_scale)
+    if (*has_scale) {
         if (int rc = scale_value(p->dtype, p->scale, p->scale_mode, scale_f)) return rc;
+        // fp32 accumulation keeps everything before its one rounding in fp32, the factor included
+        if (acc == MCCLX_ACC_F32) *scale_f = (float)p->scale;
+    }
     return MCCLX_OK;
 }
 

@@ -285,6 +285,16 @@ def test_f32acc_reduce_scatter_variant(H, U):
     H.reduce_scatter_replay(dout, din, SUM, mode=FUSED, acc=1)
     for r in range(world):
         assert np.array_equal(U.bits(dout[r]), want[r])
+    # AVG: the factor 1/world stays fp32 as well (1/7 is not a bf16 value), one rounding at the end
+    for world in (3, 7):
+        ins = [U.rand_values(rng, CH * world, BF16, scale=1e-2, specials=True) for _ in range(world)]
+        want = [np.zeros(CH, dtype=np.uint16) for _ in range(world)]
+        orc.reduce_scatter_f32acc(want, ins, AVG)
+        din = [U.to_dev(x, BF16) for x in ins]
+        dout = [torch.empty(CH, dtype=torch.bfloat16, device="cuda") for _ in range(world)]
+        H.reduce_scatter_replay(dout, din, AVG, mode=FUSED, acc=1)
+        for r in range(world):
+            U.assert_same_bits(dout[r], want[r], BF16, f"f32acc AVG world {world} rank {r}")
 
 
 @pytest.mark.parametrize("algo", [RING, TREE, BUTTERFLY])
