@@ -4,10 +4,13 @@ combinations the hand-written cases do not enumerate (a fold plan has six
 parameters, a segment five pointers with their own misalignment, a replay a
 world size, an algorithm, an op, a dtype, a wire codec and a mode)."""
 import ctypes as C
+import datetime
+import threading
 
 import numpy as np
 import pytest
 import torch
+import torch.distributed as dist
 
 from oracle import oracle as orc
 from oracle.oracle import F32, F16, BF16, SUM, AVG, MIN, MAX, PRODUCT, RING, TREE, BUTTERFLY
@@ -15,6 +18,9 @@ from oracle.oracle import F32, F16, BF16, SUM, AVG, MIN, MAX, PRODUCT, RING, TRE
 pytestmark = pytest.mark.gpu
 
 ES = {F32: 4, F16: 2, BF16: 2}
+OPS = {SUM: dist.ReduceOp.SUM, AVG: dist.ReduceOp.AVG, MIN: dist.ReduceOp.MIN, MAX: dist.ReduceOp.MAX,
+       PRODUCT: dist.ReduceOp.PRODUCT}
+TIMEOUT = datetime.timedelta(seconds=30)
 NAMES = {RING: "ring", TREE: "tree", BUTTERFLY: "butterfly"}
 
 
@@ -200,6 +206,86 @@ def reduce_scatter_case(case, rng, K, H, U):
         assert np.array_equal(U.bits(gout[r]), cat), desc + f" allgather rank {r}"
 
 
+def run_ranks(CX, world, fn):
+    store = dist.HashStore()
+    out, errs = [None] * world, [None] * world
+
+    def body(r):
+        try:
+            torch.cuda.set_device(0)
+            pg = CX._create_process_group_mccl(store, r, world, TIMEOUT)
+            out[r] = fn(r, pg)
+        except BaseException as e:  # noqa: BLE001
+            errs[r] = e
+
+    ts = [threading.Thread(target=body, args=(r,)) for r in range(world)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join(90)
+    assert not any(t.is_alive() for t in ts), "a rank thread hung"
+    return out, errs
+
+
+def collective_mix_case(case, rng, monkeypatch, CX, U):
+    world = int(rng.choice([2, 3, 4]))
+    dtype = int(rng.choice([F32, BF16]))
+    asyn = bool(rng.integers(0, 4))
+    queues = str(int(rng.integers(1, 3)))
+    chunk = int(rng.choice([int(rng.integers(1, 50)), int(rng.integers(50, 60000))]))
+    n = chunk * world
+    ntens = 3
+    steps = []
+    for _ in range(int(rng.integers(3, 10))):
+        kind = int(rng.choice([0, 0, 0, 1, 2, 3]))
+        steps.append((kind, int(rng.integers(0, ntens)), int(rng.integers(0, ntens)), int(rng.choice([SUM, MAX, MIN, AVG]))))
+    desc = f"case {case}: world {world} dtype {dtype} async {asyn} queues {queues} chunk {chunk} steps {steps}"
+    for k in ("MCCL_ALLREDUCE_ALGO", "MCCL_WIRE", "MCCL_ALLREDUCE_ASYNC", "MCCL_WIRE_DTYPE"):
+        monkeypatch.delenv(k, raising=False)
+    monkeypatch.setenv("MCCL_ASYNC_QUEUES", queues)
+    if asyn:
+        monkeypatch.setenv("MCCL_ALLREDUCE_ASYNC", "1")
+    big = [[U.rand_values(rng, n, dtype, scale=1e-2) for _ in range(ntens)] for _ in range(world)]     # world*chunk tensors
+    small = [[U.rand_values(rng, chunk, dtype, scale=1e-2) for _ in range(ntens)] for _ in range(world)]
+    def fn(r, pg):
+        B = [U.to_dev(x, dtype) for x in big[r]]
+        S = [U.to_dev(x, dtype) for x in small[r]]
+        works = []
+        for kind, i, j, op in steps:
+            o = dist.AllreduceOptions(); o.reduceOp = OPS[op]
+            if kind == 0:
+                works.append(pg.allreduce([B[i]], o))
+            elif kind == 1:
+                works.append(pg.allreduce([S[j], B[i]], o))
+            elif kind == 2:
+                ro = dist.ReduceScatterOptions(); ro.reduceOp = OPS[op]
+                works.append(pg._reduce_scatter_base(S[j], B[i], ro))
+            else:
+                works.append(pg._allgather_base(B[i], S[j]))
+        for w in works:
+            w.wait()
+        torch.cuda.current_stream().synchronize()
+        return B, S
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, (desc, errs)
+    WB = [[big[r][t].copy() for r in range(world)] for t in range(ntens)]
+    WS = [[small[r][t].copy() for r in range(world)] for t in range(ntens)]
+    for kind, i, j, op in steps:
+        if kind == 0:
+            assert orc.pg_allreduce(WB[i], dtype, op)[0] == 0
+        elif kind == 1:
+            assert orc.pg_allreduce(WS[j], dtype, op)[0] == 0
+            assert orc.pg_allreduce(WB[i], dtype, op)[0] == 0
+        elif kind == 2:
+            assert orc.reduce_scatter(WS[j], WB[i], dtype, op) == 0
+        else:
+            orc.allgather(WB[i], WS[j])
+    for r in range(world):
+        for t in range(ntens):
+            U.assert_same_bits(out[r][0][t], WB[t][r], dtype, desc + f" big {t} rank {r}")
+            U.assert_same_bits(out[r][1][t], WS[t][r], dtype, desc + f" small {t} rank {r}")
+
+
 @pytest.mark.parametrize("seed", [11, 12, 13])
 def test_random_fold_plans_segments_and_alignments(env, seed):
     K, H, L, U = env
@@ -217,3 +303,15 @@ def test_random_schedules(env, seed):
             allreduce_case(case, rng, H, U)
         else:
             reduce_scatter_case(case, rng, K, H, U)
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_random_mixes_of_collectives_on_shared_tensors_through_the_process_group(env, monkeypatch, seed):
+    """allreduce (synchronous or event-based on one or two queues, single tensors and lists),
+    reduce_scatter and allgather issued back to back on tensors they share, with no Work waited
+    on before the end: every call must see the result of the calls before it."""
+    from mccl_amd import _C as CX
+    K, H, L, U = env
+    rng = np.random.default_rng(seed)
+    for case in range(60):
+        collective_mix_case(case, rng, monkeypatch, CX, U)
