@@ -250,7 +250,7 @@ std::vector<std::string> peer_wire_probe(const std::string& mode, int world, int
                 long held = 0;
                 std::shared_ptr<std::vector<uint8_t>> previous;
                 for (int i = 0; i < rounds; ++i) {
-                    const size_t len = static_cast<size_t>(i) * 1000 + (i == 0 ? 0 : 17);  // round 0: an empty message
+                    const size_t len = static_cast<size_t>(i) * 1000 + (i == 0 ? 0 : 17);  // the first message is empty
                     auto buf = std::make_shared<std::vector<uint8_t>>(len);
                     for (size_t k = 0; k < len; ++k) (*buf)[k] = pattern(r, i, k);
                     if (mode == "kept")
@@ -261,7 +261,7 @@ std::vector<std::string> peer_wire_probe(const std::string& mode, int world, int
                     std::vector<uint8_t> got(len, 0xEE);
                     peer.recv(left, got.data(), len);
                     for (size_t k = 0; k < len; ++k)
-                        if (got[k] != pattern(left, i, k)) throw mccl::MCCLError("wrong byte in round " + std::to_string(i));
+                        if (got[k] != pattern(left, i, k)) throw mccl::MCCLError("wrong byte in message " + std::to_string(i));
                     if (mode == "kept") {
                         // our message is released once the right neighbour has taken it; it
                         // takes it before it can send us round i+1, so check one round late
