@@ -158,6 +158,17 @@ typedef struct {
  * (AllreduceAlgos.cpp:72-74); MIN and MAX keep dst on a tie or a NaN
  * (shaders.metal:65-72), so they can tell the two apart. */
 #define MCCLX_PLAN_ACC_IS_SRC 1
+/* Fan-out: the result is also written to n further destinations, in[k] ..
+ * in[k+n-1], in the form `out` has (the allgather leg of an allreduce done by
+ * the reduce itself: the owner stores its reduced chunk into every other
+ * rank's tensor instead of a second pass reading it back; with the bf16 wire
+ * the other ranks' cast of the wire copy, ProcessGroupMCCL.cpp:179-183, yields
+ * the very fp32 values the owner holds).  A destination may be one of the
+ * operands.  Sums with per-step rounding only, k + n <= MCCLX_MAX_INPUTS, `out`
+ * required, io PURE or OWN_*_F32. */
+#define MCCLX_PLAN_FANOUT_SHIFT 8
+#define MCCLX_PLAN_FANOUT_MASK 0x700
+#define MCCLX_PLAN_FANOUT(n) ((n) << MCCLX_PLAN_FANOUT_SHIFT)
 
 typedef struct {
     int32_t dtype;      /* W: MCCLX_F32 / F16 / BF16                                  */

@@ -29,6 +29,12 @@ REPLAY_STEPWISE, REPLAY_FUSED = 0, 1
 PLAN_ACC_IS_SRC = 1
 
 
+def PLAN_FANOUT(n: int) -> int:
+    """plan.flags bits: the result also goes to n further destinations, in[k .. k+n-1]."""
+    return n << 8
+
+
+
 class Seg(C.Structure):
     _fields_ = [("out", C.c_void_p), ("wire_out", C.c_void_p),
                 ("inp", C.c_void_p * MAX_INPUTS), ("count", C.c_uint64)]

@@ -16,8 +16,13 @@
 #include <torch/csrc/distributed/c10d/HashStore.hpp>
 #include <torch/csrc/distributed/c10d/Store.hpp>
 
+#include <execinfo.h>
+#include <signal.h>
+#include <unistd.h>
+
 #include <atomic>
 #include <chrono>
+#include <cstdlib>
 #include <thread>
 
 #include "backend/Errors.hpp"
@@ -39,6 +44,37 @@ void* gil_release_if_held() {
 }
 void gil_take_back(void* token) {
     if (token) PyEval_RestoreThread(static_cast<PyThreadState*>(token));
+}
+
+// MCCL_ABORT_BACKTRACE=1: when the process aborts, the native stack of the aborting
+// thread goes to stderr before the handler that was installed before runs (Python's
+// faulthandler prints the interpreter's side).  An abort raised by a library on one
+// of the backend's worker threads is otherwise anonymous.
+struct sigaction g_previous_abort_action;
+void abort_backtrace(int sig, siginfo_t* info, void* uctx) {
+    static const char head[] = "\n[MCCL] SIGABRT: native stack of the aborting thread\n";
+    (void)!write(2, head, sizeof head - 1);
+    void* frames[64];
+    const int n = backtrace(frames, 64);
+    backtrace_symbols_fd(frames, n, 2);
+    sigaction(SIGABRT, &g_previous_abort_action, nullptr);
+    if (g_previous_abort_action.sa_flags & SA_SIGINFO) {
+        if (g_previous_abort_action.sa_sigaction) g_previous_abort_action.sa_sigaction(sig, info, uctx);
+    } else if (g_previous_abort_action.sa_handler != SIG_DFL && g_previous_abort_action.sa_handler != SIG_IGN) {
+        g_previous_abort_action.sa_handler(sig);
+    }
+    raise(sig);
+}
+void install_abort_backtrace() {
+    const char* e = std::getenv("MCCL_ABORT_BACKTRACE");
+    if (!e || e[0] != '1') return;
+    void* warm[2];
+    (void)backtrace(warm, 2);  // loads the unwinder now, not inside the handler
+    struct sigaction sa;
+    sa.sa_sigaction = &abort_backtrace;
+    sigemptyset(&sa.sa_mask);
+    sa.sa_flags = SA_SIGINFO | SA_NODEFER;
+    sigaction(SIGABRT, &sa, &g_previous_abort_action);
 }
 
 // Submits n tasks; task i throws when bit i of throw_mask is set (i < 64).
@@ -284,6 +320,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.doc() = "mccl_amd native backend: c10d ProcessGroup over libmcclx";
     py::register_exception<mccl::MCCLError>(m, "MCCLError", PyExc_RuntimeError);
     mccl::set_blocking_hooks({&gil_release_if_held, &gil_take_back});
+    install_abort_backtrace();
 
     m.def("_create_process_group_mccl",
           [](const c10::intrusive_ptr<c10d::Store>& store, int rank, int size,

@@ -370,16 +370,21 @@ __device__ __forceinline__ void store16(void* base, uint32_t pack, const float (
 }
 
 // `has_out` / `has_wire`: which outputs the segment names (the pointers in `s` have
-// been advanced to the tile, so they no longer tell).
-template <class C>
+// been advanced to the tile, so they no longer tell).  `fan` (fan-out kernels): the
+// result also goes to in[K .. K+fan-1], in the form `out` has.
+template <class C, bool FAN = false>
 __device__ __forceinline__ void store_pack(const SegArgs& s, bool has_out, bool has_wire, uint32_t pack,
-                                           const float (&y)[C::E]) {
+                                           const float (&y)[C::E], int fan = 0) {
     if constexpr (C::W == MCCLX_F32 || C::kOutF32) {
-        if (has_out) {
-            u32x4 t;
+        u32x4 t;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) t[j] = __float_as_uint(y[j]);
-            MCCLX_STG(gptr<u32x4_a4>(static_cast<float*>(s.out) + pack * C::E), t);
+        for (int j = 0; j < 4; ++j) t[j] = __float_as_uint(y[j]);
+        if (has_out) MCCLX_STG(gptr<u32x4_a4>(static_cast<float*>(s.out) + pack * C::E), t);
+        if constexpr (FAN) {
+#pragma unroll
+            for (int f = 0; f < MCCLX_MAX_INPUTS - C::K; ++f)
+                if (f < fan)
+                    MCCLX_STG(gptr<u32x4_a4>(static_cast<float*>(const_cast<void*>(s.in[C::K + f])) + pack * C::E), t);
         }
     }
     if constexpr (C::W != MCCLX_F32) {
@@ -388,6 +393,11 @@ __device__ __forceinline__ void store_pack(const SegArgs& s, bool has_out, bool 
         } else {
             if (has_out) store16<C>(s.out, pack, y);
             if (has_wire) store16<C>(s.wire_out, pack, y);
+            if constexpr (FAN) {
+#pragma unroll
+                for (int f = 0; f < MCCLX_MAX_INPUTS - C::K; ++f)
+                    if (f < fan) store16<C>(const_cast<void*>(s.in[C::K + f]), pack, y);
+            }
         }
     }
 }
@@ -405,8 +415,8 @@ __device__ __forceinline__ void load_elems(const SegArgs& s, uint64_t i, float (
     v[k] = load_elem<C, k>(s, i);
     if constexpr (k + 1 < C::K) load_elems<C, k + 1>(s, i, v);
 }
-template <class C>
-__device__ __forceinline__ void fold_elem(const SegArgs& s, uint64_t i, float scale, bool has_scale) {
+template <class C, bool FAN = false>
+__device__ __forceinline__ void fold_elem(const SegArgs& s, uint64_t i, float scale, bool has_scale, int fan = 0) {
     float v[C::K];
     load_elems<C, 0>(s, i, v);
     if constexpr (C::TOPO == MCCLX_TOPO_FOLD) {
@@ -421,6 +431,11 @@ __device__ __forceinline__ void fold_elem(const SegArgs& s, uint64_t i, float sc
     float y = finish<C>(v[0], scale, has_scale);
     if constexpr (C::W == MCCLX_F32 || C::kOutF32) {
         if (s.out) gptr<float>(s.out)[i] = y;
+        if constexpr (FAN) {
+#pragma unroll
+            for (int f = 0; f < MCCLX_MAX_INPUTS - C::K; ++f)
+                if (f < fan) gptr<float>(const_cast<void*>(s.in[C::K + f]))[i] = y;
+        }
     }
     if constexpr (C::W != MCCLX_F32) {
         uint16_t h = (uint16_t)Num<C::W>::enc(y);
@@ -429,6 +444,11 @@ __device__ __forceinline__ void fold_elem(const SegArgs& s, uint64_t i, float sc
         } else {
             if (s.out) gptr<uint16_t>(s.out)[i] = h;
             if (s.wire_out) gptr<uint16_t>(s.wire_out)[i] = h;
+            if constexpr (FAN) {
+#pragma unroll
+                for (int f = 0; f < MCCLX_MAX_INPUTS - C::K; ++f)
+                    if (f < fan) gptr<uint16_t>(const_cast<void*>(s.in[C::K + f]))[i] = h;
+            }
         }
     }
 }
@@ -436,9 +456,9 @@ __device__ __forceinline__ void fold_elem(const SegArgs& s, uint64_t i, float sc
 // U packets per lane: all loads first, then arithmetic, then stores.  `s` points
 // at the tile's first packet; pk[] are packet indices inside the tile, so every
 // address is a uniform 64-bit base plus a 32-bit lane offset.
-template <class C, int U>
+template <class C, int U, bool FAN = false>
 __device__ __forceinline__ void fold_packs(const SegArgs& s, bool has_out, bool has_wire, const uint32_t (&pk)[U],
-                                           float scale, bool has_scale) {
+                                           float scale, bool has_scale, int fan = 0) {
     RawPack raw[C::K][U];
     load_all<C, 0, U>(s, pk, raw);
 #pragma unroll
@@ -449,7 +469,7 @@ __device__ __forceinline__ void fold_packs(const SegArgs& s, bool has_out, bool 
         float acc[C::E];
         combine<C>(col, acc);
         finish_pack<C>(acc, scale, has_scale);
-        store_pack<C>(s, has_out, has_wire, pk[u], acc);
+        store_pack<C, FAN>(s, has_out, has_wire, pk[u], acc, fan);
     }
 }
 
@@ -471,7 +491,7 @@ __device__ __forceinline__ uint32_t head_elems(const SegArgs& s) {
 
 // Every pointer of the segment moved `elems` elements on (null outputs become
 // garbage: the caller keeps their presence in flags).
-template <class C>
+template <class C, bool FAN = false>
 __device__ __forceinline__ SegArgs advanced(const SegArgs& s, uint64_t elems) {
     SegArgs t;
     const uint64_t b2 = elems * 2, b4 = elems * 4;
@@ -479,8 +499,14 @@ __device__ __forceinline__ SegArgs advanced(const SegArgs& s, uint64_t elems) {
     t.out = static_cast<char*>(s.out) + (out_f32 ? b4 : b2);
     t.wire_out = static_cast<char*>(s.wire_out) + b2;
 #pragma unroll
-    for (int k = 0; k < MCCLX_MAX_INPUTS; ++k)
-        t.in[k] = (k < C::K) ? static_cast<const char*>(s.in[k]) + (C::in_is_f32(k) ? b4 : b2) : nullptr;
+    for (int k = 0; k < MCCLX_MAX_INPUTS; ++k) {
+        if (k < C::K)
+            t.in[k] = static_cast<const char*>(s.in[k]) + (C::in_is_f32(k) ? b4 : b2);
+        else if constexpr (FAN)
+            t.in[k] = static_cast<const char*>(s.in[k]) + (out_f32 ? b4 : b2);  // a further destination
+        else
+            t.in[k] = nullptr;
+    }
     t.count = 0;
     return t;
 }
@@ -491,9 +517,9 @@ __device__ __forceinline__ SegArgs advanced(const SegArgs& s, uint64_t elems) {
 // load is kept short -- a block lives for about 2 us and eight waves per SIMD
 // share one scalar unit, so every scalar instruction in front of the loads is
 // paid eight times over.
-template <class C>
+template <class C, bool FAN = false>
 __device__ __forceinline__ void fold_tile(const SegArgs& s, float scale, bool has_scale, uint64_t first,
-                                          bool do_edges) {
+                                          bool do_edges, int fan = 0) {
     constexpr int U = C::U;
     const uint32_t tid = threadIdx.x;
     constexpr int kB = C::BLOCK;
@@ -501,24 +527,24 @@ __device__ __forceinline__ void fold_tile(const SegArgs& s, float scale, bool ha
     const uint64_t P = (s.count - head) / C::E;
     const bool has_out = s.out != nullptr, has_wire = s.wire_out != nullptr;
     if (first < P) {
-        const SegArgs t = advanced<C>(s, head + first * C::E);
+        const SegArgs t = advanced<C, FAN>(s, head + first * C::E);
         const uint64_t left = P - first;
         if (left >= (uint64_t)U * kB) {
             uint32_t pk[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) pk[u] = (uint32_t)u * kB + tid;
-            fold_packs<C, U>(t, has_out, has_wire, pk, scale, has_scale);
+            fold_packs<C, U, FAN>(t, has_out, has_wire, pk, scale, has_scale, fan);
         } else {
             for (uint32_t p = tid; p < (uint32_t)left; p += kB) {
                 uint32_t one[1] = {p};
-                fold_packs<C, 1>(t, has_out, has_wire, one, scale, has_scale);
+                fold_packs<C, 1, FAN>(t, has_out, has_wire, one, scale, has_scale, fan);
             }
         }
     }
     if (do_edges) {
-        if (tid < head) fold_elem<C>(s, tid, scale, has_scale);
+        if (tid < head) fold_elem<C, FAN>(s, tid, scale, has_scale, fan);
         const uint64_t i = head + P * C::E + tid;  // fewer than E <= 8 elements remain
-        if (i < s.count) fold_elem<C>(s, i, scale, has_scale);
+        if (i < s.count) fold_elem<C, FAN>(s, i, scale, has_scale, fan);
     }
 }
 
@@ -548,7 +574,7 @@ __device__ __forceinline__ void fetch_together(SegArgs& s, float& scale, int32_t
 // kernel with more starts 768 blocks at launch instead of 1024 and streams
 // 2-4 % slower.  Six registers are set aside on top of what the code uses (VCC,
 // flat scratch, XNACK mask), so the code itself has 74.
-template <class C>
+template <class C, bool FAN = false>
 __device__ __forceinline__ void fold_few_body(const FewArgs& a) {
 #if MCCLX_TUNE_TIMELINE
     const uint64_t t_start = wall_clock64();
@@ -557,7 +583,9 @@ __device__ __forceinline__ void fold_few_body(const FewArgs& a) {
     float scale = a.scale;
     int32_t has_scale = a.has_scale;
     uint32_t grid = gridDim.x;
-    fetch_together<C::K>(s, scale, has_scale, grid);
+    fetch_together<FAN ? MCCLX_MAX_INPUTS : C::K>(s, scale, has_scale, grid);
+    int32_t fan = 0;
+    if constexpr (FAN) fan = a.fan;
 #if MCCLX_TUNE_TIMELINE
     const uint64_t t_args = wall_clock64();
 #endif
@@ -566,11 +594,11 @@ __device__ __forceinline__ void fold_few_body(const FewArgs& a) {
     // workgroups go to the XCDs round robin: block b runs on XCD b % N
     const uint32_t per = grid / MCCLX_TUNE_XCD;  // the grid is a multiple of N
     const uint32_t tile = (blockIdx.x % MCCLX_TUNE_XCD) * per + blockIdx.x / MCCLX_TUNE_XCD;
-    fold_tile<C>(s, scale, has_scale != 0, (uint64_t)tile * span, tile == 0);
+    fold_tile<C, FAN>(s, scale, has_scale != 0, (uint64_t)tile * span, tile == 0, fan);
 #else
     // one tile per block, no loop: the launch sizes the grid to the longest segment
     (void)grid;
-    fold_tile<C>(s, scale, has_scale != 0, (uint64_t)blockIdx.x * span, blockIdx.x == 0);
+    fold_tile<C, FAN>(s, scale, has_scale != 0, (uint64_t)blockIdx.x * span, blockIdx.x == 0, fan);
 #endif
 #if MCCLX_TUNE_TIMELINE
     if (a.timeline && threadIdx.x == 0) {
@@ -595,6 +623,10 @@ template <class C>
 __global__ void __launch_bounds__(C::BLOCK) MCCLX_SGPR_CAP fold_few_kernel(FewArgs a) { fold_few_body<C>(a); }
 template <class C>
 __global__ void __launch_bounds__(C::BLOCK) fold_few_wide_kernel(FewArgs a) { fold_few_body<C>(a); }
+// Fan-out form: the result also goes to in[K .. K+fan-1] (the other ranks' tensors: the
+// allgather leg of an allreduce done by the reduce itself, stores instead of a second pass).
+template <class C>
+__global__ void __launch_bounds__(C::BLOCK) fold_few_fan_kernel(FewArgs a) { fold_few_body<C, true>(a); }
 
 // A value that is the same in every lane, moved to scalar registers.  The
 // compiler cannot always prove it (a quotient comes out of the vector ALU), and
@@ -614,7 +646,7 @@ __device__ __forceinline__ P* uniptr(P* p) {
 // blockIdx.x + gridDim.x, ...  (one item per block unless the grid is capped).
 // The loop bound is fixed at launch, so every wave exits.  total_items < 2^31
 // (checked by the host).
-template <class C>
+template <class C, bool FAN = false>
 __device__ __forceinline__ void fold_table_body(const TableArgs& a) {
     const uint64_t span = (uint64_t)C::U * C::BLOCK;
     const uint32_t total = (uint32_t)a.total_items;
@@ -645,10 +677,10 @@ __device__ __forceinline__ void fold_table_body(const TableArgs& a) {
         s.out = uniptr(d->out);
         s.wire_out = uniptr(d->wire_out);
 #pragma unroll
-        for (int k = 0; k < MCCLX_MAX_INPUTS; ++k) s.in[k] = (k < C::K) ? uniptr(d->in[k]) : nullptr;
+        for (int k = 0; k < MCCLX_MAX_INPUTS; ++k) s.in[k] = (k < C::K || FAN) ? uniptr(d->in[k]) : nullptr;
         s.count = uni64(d->count);
         // one tile: packets [tile*span, tile*span + span); tile 0 also owns the tail
-        fold_tile<C>(s, a.scale, a.has_scale != 0, (uint64_t)tile * span, tile == 0);
+        fold_tile<C, FAN>(s, a.scale, a.has_scale != 0, (uint64_t)tile * span, tile == 0, FAN ? a.fan : 0);
     }
 }
 
@@ -656,6 +688,13 @@ template <class C>
 __global__ void __launch_bounds__(C::BLOCK) MCCLX_SGPR_CAP fold_table_kernel(TableArgs a) { fold_table_body<C>(a); }
 template <class C>
 __global__ void __launch_bounds__(C::BLOCK) fold_table_wide_kernel(TableArgs a) { fold_table_body<C>(a); }
+template <class C>
+__global__ void __launch_bounds__(C::BLOCK) fold_table_fan_kernel(TableArgs a) { fold_table_body<C, true>(a); }
+
+// Plans with a fan-out form (host mirror: fan_plan_ok).
+template <class C>
+constexpr bool kFanPlan = C::OP == MCCLX_SUM && C::ACC == MCCLX_ACC_STEP && C::K >= 2 && C::K < MCCLX_MAX_INPUTS &&
+                          C::IO != MCCLX_IO_OUT_F32;
 
 // ----------------------------------------------------------------- dispatch
 
@@ -688,6 +727,33 @@ static constexpr size_t wide_lds_bytes() { return 0; }
 template <class C>
 static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
     const uint64_t span = (uint64_t)C::U * C::BLOCK * C::E;  // elements per block iteration
+    if (lp.fan > 0) {
+        if constexpr (!kFanPlan<C>) {
+            return hipErrorInvalidValue;
+        } else {
+            if (lp.fan > MCCLX_MAX_INPUTS - C::K) return hipErrorInvalidValue;
+            if (lp.table) {
+                TableArgs a = *lp.table;
+                a.fan = lp.fan;
+                uint32_t grid = (uint32_t)(a.total_items < lp.max_blocks ? a.total_items : lp.max_blocks);
+                if (grid == 0) return hipSuccess;
+                fold_table_fan_kernel<C><<<dim3(grid), dim3(C::BLOCK), 0, st>>>(a);
+            } else {
+                FewArgs a = *lp.few;
+                a.fan = lp.fan;
+                uint64_t maxc = 0;
+                for (int i = 0; i < a.nseg; ++i) maxc = a.seg[i].count > maxc ? a.seg[i].count : maxc;
+                if (maxc == 0) return hipSuccess;
+                uint64_t gx = (maxc + span - 1) / span;
+                if (gx >> 31) return hipErrorInvalidValue;
+#if MCCLX_TUNE_TIMELINE
+                a.timeline = nullptr;
+#endif
+                fold_few_fan_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(C::BLOCK), 0, st>>>(a);
+            }
+            return hipGetLastError();
+        }
+    }
     if (lp.table) {
         TableArgs a = *lp.table;
         uint32_t grid = (uint32_t)(a.total_items < lp.max_blocks ? a.total_items : lp.max_blocks);
@@ -747,6 +813,11 @@ static bool key_is_wide(const PlanKey& key) { return key_pack_elems(key) == 8 &&
 int plan_block(const PlanKey& key) {
     const bool decode = key.k == 1 && key.io == MCCLX_IO_OUT_F32;
     return key_is_wide(key) ? kWideBlock : ((key.dtype == MCCLX_F32 && key.k >= 2) || decode ? MCCLX_TUNE_F32_BLOCK : kBlock);
+}
+
+bool fan_plan_ok(const PlanKey& key) {
+    return key.op == MCCLX_SUM && key.acc == MCCLX_ACC_STEP && key.k >= 2 && key.k < MCCLX_MAX_INPUTS &&
+           key.io != MCCLX_IO_OUT_F32;
 }
 
 int plan_unroll(const PlanKey& key) {

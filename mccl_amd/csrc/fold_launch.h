@@ -42,6 +42,7 @@ struct FewArgs {
     float scale;        // the constant as the fp32 value the kernel multiplies by
     int32_t has_scale;
     int32_t nseg;
+    int32_t fan;        // further destinations of the result, in[k .. k+fan-1] (fan-out kernels only)
 #if MCCLX_TUNE_TIMELINE
     TimelineRecord* timeline;  // this launch's records, one per block (x fastest, then y), or null
 #endif
@@ -56,6 +57,7 @@ struct TableArgs {
     uint32_t nseg;
     float scale;
     int32_t has_scale;
+    int32_t fan;                 // further destinations of the result, in[k .. k+fan-1] (fan-out kernels only)
 };
 
 // Kernel-side operator codes beyond the public MCCLX_* ones: MIN / MAX with the
@@ -70,7 +72,10 @@ struct LaunchParams {
     const FewArgs* few = nullptr;      // exactly one of few / table is set
     const TableArgs* table = nullptr;
     uint32_t max_blocks = 0;           // cap on the grid (persistent sizing)
+    int fan = 0;                       // > 0: the fan-out form of the kernel (plans in fan_plan_ok only)
 };
+// Plans that have a fan-out form: sums with per-step rounding, 2..7 operands.
+bool fan_plan_ok(const PlanKey& key);
 
 // Packets-per-lane unroll and threads per block the kernel template uses for this plan.
 int plan_unroll(const PlanKey& key);

@@ -196,9 +196,11 @@ int normalize_op(int op, int* out) {
     }
 }
 
-int check_plan(const mcclx_plan* p, mcclx::PlanKey* key, float* scale_f, int* has_scale) {
+int check_plan(const mcclx_plan* p, mcclx::PlanKey* key, float* scale_f, int* has_scale, int* fan) {
     if (!p) return fail(MCCLX_ERR_INVALID, "plan is null");
-    if (p->flags & ~MCCLX_PLAN_ACC_IS_SRC) return fail(MCCLX_ERR_INVALID, "plan.flags=%d has unknown bits", p->flags);
+    if (p->flags & ~(MCCLX_PLAN_ACC_IS_SRC | MCCLX_PLAN_FANOUT_MASK))
+        return fail(MCCLX_ERR_INVALID, "plan.flags=%d has unknown bits", p->flags);
+    *fan = (p->flags & MCCLX_PLAN_FANOUT_MASK) >> MCCLX_PLAN_FANOUT_SHIFT;
     if (!dtype_ok(p->dtype))
         return fail(MCCLX_ERR_UNSUPPORTED, "No kernel for dtype code %d", p->dtype);
     if (p->k < 1 || p->k > MCCLX_MAX_INPUTS)
@@ -227,6 +229,11 @@ int check_plan(const mcclx_plan* p, mcclx::PlanKey* key, float* scale_f, int* ha
         op = (op == MCCLX_MIN) ? mcclx::MCCLX_MIN_ACC_SRC : mcclx::MCCLX_MAX_ACC_SRC;
     int acc = (p->dtype == MCCLX_F32) ? MCCLX_ACC_STEP : p->acc;  // fp32 has no rounding to skip
     *key = mcclx::PlanKey{p->dtype, p->io, p->k, (p->k >= 4) ? p->topo : MCCLX_TOPO_FOLD, op, acc};
+    if (*fan && (!mcclx::fan_plan_ok(*key) || p->k + *fan > MCCLX_MAX_INPUTS))
+        return fail(MCCLX_ERR_UNSUPPORTED,
+                    "fan-out (%d further destinations) needs a sum with per-step rounding, an output of the "
+                    "operands' form or fp32 next to an fp32 operand, and k + fan <= %d (k=%d)",
+                    *fan, MCCLX_MAX_INPUTS, p->k);
     *has_scale = p->scale_mode != MCCLX_SCALE_NONE;
     *scale_f = 1.0f;
     if (*has_scale) {
@@ -267,7 +274,7 @@ int check_range(const void* p, uint64_t nbytes, const char* what, uint32_t seg) 
     return MCCLX_OK;
 }
 
-int check_segs(mcclx_ctx* ctx, const mcclx::PlanKey& key, const mcclx_seg* segs, uint32_t nseg) {
+int check_segs(mcclx_ctx* ctx, const mcclx::PlanKey& key, const mcclx_seg* segs, uint32_t nseg, int fan) {
     if (!segs && nseg) return fail(MCCLX_ERR_INVALID, "segment array is null");
     const bool out_f32 = key.dtype == MCCLX_F32 || key.io != MCCLX_IO_PURE;
     for (uint32_t s = 0; s < nseg; ++s) {
@@ -288,6 +295,16 @@ int check_segs(mcclx_ctx* ctx, const mcclx::PlanKey& key, const mcclx_seg* segs,
         if (g.wire_out && (uintptr_t)g.wire_out % 2)
             return fail(MCCLX_ERR_INVALID, "segment %u: wire_out=%p is not element aligned", s,
                         g.wire_out);
+        if (fan && !g.out) return fail(MCCLX_ERR_INVALID, "segment %u: fan-out needs `out`", s);
+        for (int f = 0; f < fan; ++f) {
+            const void* d = g.in[key.k + f];
+            if (!d) return fail(MCCLX_ERR_INVALID, "segment %u: fan-out destination in[%d] is null", s, key.k + f);
+            if ((uintptr_t)d % (out_f32 ? 4 : 2))
+                return fail(MCCLX_ERR_INVALID, "segment %u: fan-out destination in[%d]=%p is not element aligned", s,
+                            key.k + f, d);
+            if (ctx->validate)
+                if (int rc = check_range(d, g.count * (out_f32 ? 4 : 2), "fan-out destination", s)) return rc;
+        }
         if (ctx->validate) {
             for (int i = 0; i < key.k; ++i)
                 if (int rc = check_range(g.in[i], g.count * (in_is_f32(key, i) ? 4 : 2), "in", s))
@@ -378,9 +395,10 @@ int stage_table(mcclx_ctx* ctx, const void* bytes, size_t nbytes, void** dev, Ta
 
 // Descriptors in the kernel arguments (nseg <= kFewSegs).
 int launch_by_value(mcclx_ctx* ctx, const mcclx::PlanKey& key, float scale_f, int has_scale,
-                    const mcclx_seg* segs, uint32_t nseg) {
+                    const mcclx_seg* segs, uint32_t nseg, int fan) {
     mcclx::LaunchParams lp;
     lp.max_blocks = ctx->max_blocks;
+    lp.fan = fan;
     mcclx::FewArgs a;
     memset(&a, 0, sizeof a);
     for (uint32_t s = 0; s < nseg; ++s) memcpy(&a.seg[s], &segs[s], sizeof(mcclx_seg));
@@ -398,9 +416,9 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
     if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
     mcclx::PlanKey key;
     float scale_f;
-    int has_scale;
-    if (int rc = check_plan(plan, &key, &scale_f, &has_scale)) return rc;
-    if (int rc = check_segs(ctx, key, segs, nseg)) return rc;
+    int has_scale, fan;
+    if (int rc = check_plan(plan, &key, &scale_f, &has_scale, &fan)) return rc;
+    if (int rc = check_segs(ctx, key, segs, nseg, fan)) return rc;
     if (nseg == 0) return MCCLX_OK;
     DeviceGuard guard(ctx->device);
     if (!guard.ok) return fail(MCCLX_ERR_HIP, "hipSetDevice(%d) failed", ctx->device);
@@ -420,7 +438,7 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
         }
         by_value = longest * nseg <= 4 * total + 64;
     }
-    if (by_value) return launch_by_value(ctx, key, scale_f, has_scale, segs, nseg);
+    if (by_value) return launch_by_value(ctx, key, scale_f, has_scale, segs, nseg, fan);
 
     // descriptor table: segs, then nseg+1 work-item prefix sums
     std::lock_guard<std::mutex> lk(ctx->mu);
@@ -464,6 +482,7 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
     t.scale = scale_f;
     t.has_scale = has_scale;
     lp.table = &t;
+    lp.fan = fan;
     hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
     if (e != hipSuccess) return launch_error(e, key);
     ++ctx->launches;
@@ -591,13 +610,13 @@ int mcclx_fold_batched_noalloc(mcclx_ctx* ctx, const mcclx_plan* plan, const mcc
                     nseg, MCCLX_NOALLOC_MAX_SEGS);
     mcclx::PlanKey key;
     float scale_f;
-    int has_scale;
-    if (int rc = check_plan(plan, &key, &scale_f, &has_scale)) return rc;
-    if (int rc = check_segs(ctx, key, segs, nseg)) return rc;
+    int has_scale, fan;
+    if (int rc = check_plan(plan, &key, &scale_f, &has_scale, &fan)) return rc;
+    if (int rc = check_segs(ctx, key, segs, nseg, fan)) return rc;
     if (nseg == 0) return MCCLX_OK;
     DeviceGuard guard(ctx->device);
     if (!guard.ok) return fail(MCCLX_ERR_HIP, "hipSetDevice(%d) failed", ctx->device);
-    if (nseg <= (uint32_t)mcclx::kFewSegs) return launch_by_value(ctx, key, scale_f, has_scale, segs, nseg);
+    if (nseg <= (uint32_t)mcclx::kFewSegs) return launch_by_value(ctx, key, scale_f, has_scale, segs, nseg, fan);
 
     uint64_t total = 0, uniform = mcclx::items_for(key, segs[0].count);
     for (uint32_t s = 0; s < nseg; ++s) {
@@ -645,6 +664,7 @@ int mcclx_fold_batched_noalloc(mcclx_ctx* ctx, const mcclx_plan* plan, const mcc
     mcclx::LaunchParams lp;
     lp.max_blocks = ctx->max_blocks;
     lp.table = &t;
+    lp.fan = fan;
     hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
     if (e != hipSuccess) return launch_error(e, key);
     ++ctx->launches;

@@ -214,7 +214,27 @@ struct Phases {
     std::vector<mcclx_seg> enc_segs, dec_segs;
     std::vector<FoldPass> folds;  // one pass, or a chain of passes when the world is wider than one fold
     std::vector<mcclx_copy_desc> copies;
+    int fan = 0;  // > 0: the fold itself stores every reduced chunk into the other ranks' tensors
+                  // (in[k .. k+fan-1] of its segments); there is no allgather launch then
 };
+
+// A sum over so few ranks that operands and destinations fit one segment (k ranks +
+// k-1 other tensors <= MCCLX_MAX_INPUTS, i.e. up to 4 ranks): the owner's fold writes
+// the result to everybody -- what the allgather leg and the final cast would
+// deliver (AllreduceAlgos.cpp:77-86,116-131,185-200, ProcessGroupMCCL.cpp:179-183: the
+// other ranks' cast of the bf16 result gives the very fp32 values the owner holds).
+// MCCLX_FANOUT=0 keeps the separate allgather launch.
+int fan_of(const mcclx_replay* r) {
+    static const bool enabled = [] {
+        const char* e = getenv("MCCLX_FANOUT");
+        return !(e && e[0] == '0');
+    }();
+    const bool sum = r->op == MCCLX_SUM || r->op == MCCLX_AVG;
+    const bool wire = r->wire_bf16 && r->dtype == MCCLX_F32;
+    const bool step = r->acc == MCCLX_ACC_STEP || (r->dtype == MCCLX_F32 && !wire);  // fp32 has no rounding to skip
+    if (!enabled || !sum || !step || r->world < 2 || 2 * r->world - 1 > MCCLX_MAX_INPUTS) return 0;
+    return r->world - 1;
+}
 
 // MIN / MAX / PRODUCT over the wire codec: the fold kernels mix fp32 and bf16
 // operands for sums only, so for these ops every rank encodes its WHOLE tensor
@@ -281,6 +301,8 @@ void plan_phases(const mcclx_replay* r, const Layout& L, Phases& ph) {
     }
     mcclx_plan& fold = ph.folds[0].plan;
     if (r->algo == MCCLX_ALGO_TREE) fold.topo = MCCLX_TOPO_BINOMIAL;
+    ph.fan = fan_of(r);
+    if (ph.fan) fold.flags |= MCCLX_PLAN_FANOUT(ph.fan);
     if (L.wire && !all_on_wire(r)) {  // the owner's operand is read as fp32 and encoded in registers
         if (r->algo == MCCLX_ALGO_TREE)
             fold.io = MCCLX_IO_OWN_FIRST_F32;
@@ -357,9 +379,14 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
             s.out = r->tensors[0];
             s.in[0] = r->tensors[0];
             for (int q = 1; q < N; ++q) s.in[q] = L.wire ? wire_of(q) : r->tensors[q];
-            if (L.wire) s.wire_out = wire_of(0);
+            if (ph.fan) {  // rank 0's fold hands the result to ranks 1..N-1 itself
+                for (int q = 1; q < N; ++q) s.in[N + q - 1] = r->tensors[q];
+            } else if (L.wire) {
+                s.wire_out = wire_of(0);
+            }
         }
         ph.folds[0].segs.push_back(s);
+        if (ph.fan) return;
         for (int q = bf16_only ? 0 : 1; q < N; ++q) {
             if (L.wire) {  // broadcast of the bf16 result + the final cast on every rank
                 mcclx_seg g = z;
@@ -415,8 +442,14 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
             mcclx_seg s = z;
             s.count = (uint64_t)c[ch].elem_count;
             s.out = dest;
-            if (L.wire && !bf16_only) s.wire_out = at(wire_of(o), (uint64_t)c[ch].elem_start * 2);
             for (int j = 0; j < N; ++j) s.in[j] = ops[(size_t)j];
+            if (ph.fan) {  // the owner's fold hands the reduced chunk to every other rank itself
+                int f = 0;
+                for (int q = 0; q < N; ++q)
+                    if (q != o) s.in[N + f++] = at(r->tensors[q], (uint64_t)c[ch].elem_start * ts);
+            } else if (L.wire && !bf16_only) {
+                s.wire_out = at(wire_of(o), (uint64_t)c[ch].elem_start * 2);
+            }
             ph.folds[0].segs.push_back(s);
             continue;
         }
@@ -440,6 +473,7 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
     // allgather leg (AllreduceAlgos.cpp:77-86,185-200): every other rank gets
     // the owner's reduced chunk; with the wire codec it arrives as bf16 and is
     // cast on arrival (ProcessGroupMCCL.cpp:179-183).
+    if (ph.fan) return;  // done by the folds
     for (int ch = 0; ch < N; ++ch) {
         if (c[ch].elem_count == 0) continue;
         int o = owner_of(ch);

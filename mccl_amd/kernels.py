@@ -226,8 +226,10 @@ def make_seg(out=0, wire_out=0, inputs=(), count=0) -> L.Seg:
 
 
 def make_plan(dtype, k, io=L.IO_PURE, topo=L.TOPO_FOLD, op=L.SUM, acc=L.ACC_STEP,
-              scale_mode=L.SCALE_NONE, scale=0.0, flags=0) -> L.Plan:
-    return L.Plan(dtype, io, k, topo, op, acc, scale_mode, flags, scale)
+              scale_mode=L.SCALE_NONE, scale=0.0, flags=0, fanout=0) -> L.Plan:
+    """`fanout` = n: the result is also stored to n further destinations, which the segment
+    names in inputs[k .. k+n-1]."""
+    return L.Plan(dtype, io, k, topo, op, acc, scale_mode, flags | L.PLAN_FANOUT(fanout), scale)
 
 
 # ---- tensor variants (MetalKernels.hpp:14-43) ------------------------------

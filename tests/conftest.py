@@ -5,6 +5,8 @@ import pytest
 
 # libmcclx checks every launch's pointers against their allocations when this is set
 os.environ.setdefault("MCCLX_VALIDATE", "1")
+# should the process ever abort, the extension prints the native stack of the thread that did it
+os.environ.setdefault("MCCL_ABORT_BACKTRACE", "1")
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 for p in (ROOT, os.path.join(ROOT, "tests")):

@@ -391,7 +391,7 @@ def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypat
     # together, 3 launches; two queues -- two at once on either queue, behind them buckets 4 and
     # 6 together and bucket 5, 6 launches.  A rank thread that is held up may split a group.
     assert (3 if queues == 1 else 6) <= l1 - l0 < len(sizes), "buckets were coalesced"
-    assert k1 - k0 == 3 * (l1 - l0), "a launch of several buckets is encode + fold + cast, once"
+    assert k1 - k0 == 2 * (l1 - l0), "a launch of several buckets is encode + fold (which also hands out the result), once"
     assert all(all(out[r][2]) for r in range(world)), "a Work was complete when allreduce returned"
 
 

@@ -10,6 +10,7 @@ Stronger than the reference's allclose checks where arithmetic allows: ranks
 must agree bit for bit, and with two ranks (one commutative add per element) the
 synchronised gradient must equal the oracle's allreduce of the local gradients."""
 import datetime
+import gc
 import threading
 
 import numpy as np
@@ -51,6 +52,9 @@ def run_default_groups(world, fn):
                 with torch.autograd.set_multithreading_enabled(False):
                     out[r] = fn(r, world)
             finally:
+                # DDP modules sit in reference cycles: collect them here, on the rank's own thread and
+                # while its group exists, not whenever and wherever the collector next runs
+                gc.collect()
                 dist.destroy_process_group()
         except BaseException as e:  # noqa: BLE001
             errs[r] = e

@@ -432,3 +432,84 @@ def test_scale_after_a_fold_keeps_the_sign_of_zero(K, U, dtype, op):
                 assert np.array_equal(U.bits(out), v[0]), (op, k, scale)
             else:
                 U.assert_same_bits(out, v[0], dtype, f"dtype {dtype} op {op} k {k} scale {scale}")
+
+
+@pytest.mark.parametrize("kind", ["f32", "bf16", "f16", "own_first", "own_last"])
+def test_fan_out_writes_the_result_to_every_destination(K, U, kind):
+    """MCCLX_PLAN_FANOUT(n): what `out` receives also goes to in[k .. k+n-1] -- the owner of a
+    chunk handing the reduced values to every other rank (AllreduceAlgos.cpp:77-86,185-200)
+    without a second pass.  Every k and n that fit a segment, both topologies, misaligned
+    destinations, a destination that is one of the operands, by-value and table launches."""
+    rng = np.random.default_rng(len(kind) * 7)
+    dtype = {"f32": F32, "bf16": BF16, "f16": F16}.get(kind, BF16)
+    io = {"own_first": L().IO_OWN_FIRST_F32, "own_last": L().IO_OWN_LAST_F32}.get(kind, L().IO_PURE)
+    odt = F32 if (dtype == F32 or io != L().IO_PURE) else dtype
+    es = {F32: 4, F16: 2, BF16: 2}
+    for k in range(2, 8):
+        for fan in range(1, 9 - k):
+            for binomial in ((False, True) if (k >= 4 and kind != "own_last") else (False,)):
+                nseg = int(rng.choice([1, 3, 40]))
+                segs, checks, keep = [], [], []
+                for s in range(nseg):
+                    n = int(rng.integers(1, 30000 if nseg < 10 else 3000))
+                    ins, ptrs, dev = [], [], []
+                    for j in range(k):
+                        f32_in = dtype == F32 or (kind == "own_first" and j == 0) or (kind == "own_last" and j == k - 1)
+                        dt = F32 if f32_in else dtype
+                        off = int(rng.integers(0, 5))
+                        a = U.rand_values(rng, n + off + 4, dt, scale=1e-2, specials=(dt != F16))
+                        t = U.to_dev(a, dt)
+                        ins.append((np.ascontiguousarray(a[off:off + n]), dt))
+                        dev.append(t)
+                        ptrs.append(t.data_ptr() + off * es[dt])
+                    ops = [orc.encode_bf16(a) if (dt == F32 and dtype == BF16) else a.copy() for a, dt in ins]
+                    res = oracle_fold(ops, dtype, binomial and k >= 4, 1.0 / 3, orc.SCALE_VIEW)
+                    want = orc.decode_bf16(res) if (odt == F32 and dtype == BF16) else res
+                    outs = []
+                    for f in range(fan + 1):
+                        off = int(rng.integers(0, 5))
+                        t = torch.full((n + off + 4,), 3.0, dtype=U.TORCH_DT[odt], device="cuda")
+                        outs.append((t, off))
+                    # one destination may be an operand of the output's form (reduced in place)
+                    same_form = [j for j, (a, dt) in enumerate(ins) if dt == odt]
+                    if same_form and rng.integers(0, 2):
+                        j = int(rng.choice(same_form))
+                        outs[-1] = (dev[j], (ptrs[j] - dev[j].data_ptr()) // es[odt])
+                    dest = [t.data_ptr() + off * es[odt] for t, off in outs]
+                    segs.append(K.make_seg(dest[0], 0, ptrs + dest[1:], n))
+                    checks.append((outs, n, want))
+                    keep.append(dev)
+                plan = K.make_plan(dtype, k, io=io, topo=L().TOPO_BINOMIAL if binomial else L().TOPO_FOLD,
+                                   scale_mode=L().SCALE_VIEW, scale=1.0 / 3, fanout=fan)
+                torch.cuda.synchronize()
+                K._q(None).fold(plan, segs)
+                K.hip_sync()
+                for outs, n, want in checks:
+                    for f, (t, off) in enumerate(outs):
+                        what = f"{kind} k={k} fan={fan} binomial={binomial} nseg={nseg} destination {f}"
+                        if odt == F16:
+                            assert np.array_equal(U.bits(t[off:off + n]), want), what
+                        else:
+                            U.assert_same_bits(t[off:off + n], want, odt, what)
+                        if t.numel() == n + off + 4 and float(t[:1].float().cpu()) == 3.0:   # a fresh buffer: guards intact
+                            assert torch.all(t[:off].float() == 3.0) and torch.all(t[off + n:].float() == 3.0), what
+
+
+def test_fan_out_validation(K):
+    q = K._q(None)
+    t = torch.zeros(64, device="cuda")
+    seg = lambda k, fan: [K.make_seg(t.data_ptr(), 0, [t.data_ptr()] * min(8, k + fan), 16)]
+    for plan, fan, k, frag in ((K.make_plan(F32, 5, fanout=4), 4, 5, "k + fan <= 8"),
+                               (K.make_plan(F32, 3, op=orc.MAX, fanout=2), 2, 3, "needs a sum"),
+                               (K.make_plan(BF16, 3, acc=L().ACC_F32, fanout=2), 2, 3, "per-step rounding"),
+                               (K.make_plan(BF16, 2, io=L().IO_OUT_F32, fanout=1), 1, 2, "fan-out"),
+                               (K.make_plan(F32, 1, fanout=1), 1, 1, "fan-out")):
+        with pytest.raises(Exception) as e:
+            q.fold(plan, seg(k, fan))
+        assert frag in str(e.value), str(e.value)
+    with pytest.raises(Exception) as e:                                 # a destination is missing
+        q.fold(K.make_plan(F32, 2, fanout=2), [K.make_seg(t.data_ptr(), 0, [t.data_ptr()] * 3, 16)])
+    assert "fan-out destination in[3] is null" in str(e.value)
+    with pytest.raises(Exception) as e:                                 # fan-out without `out`
+        q.fold(K.make_plan(BF16, 2, fanout=1), [K.make_seg(0, t.data_ptr(), [t.data_ptr()] * 3, 16)])
+    assert "fan-out needs `out`" in str(e.value)

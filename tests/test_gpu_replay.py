@@ -363,9 +363,12 @@ def test_copy_batched_many_small_and_a_few_large(K, U):
 
 
 def test_launch_counts_of_the_fused_schedules(H, K, U):
-    """What "fused" means in launches: butterfly over the wire = encode + fold + cast (3), for any
-    reduce op; without the wire 1 fold + the allgather copies; a list of 200 tree messages = 1 fold
-    + 1 copy launch; the stepwise replay of the same butterfly issues the reference's sequence."""
+    """What "fused" means in launches.  Up to four ranks a sum needs no allgather launch: the
+    owner's fold stores the reduced chunk into every rank's tensor, so butterfly over the wire =
+    encode + fold (2) and without the wire one fold (1); the other reduce ops, and five ranks or
+    more, keep the separate cast / copy launch (3, or 1 fold + the allgather copies); a list of
+    200 tree messages = 1 launch; the stepwise replay of the same butterfly issues the
+    reference's sequence."""
     from mccl_amd import _lib as L
     q = K._q(None)
     world, n = 3, 300_000
@@ -379,14 +382,19 @@ def test_launch_counts_of_the_fused_schedules(H, K, U):
     mk = lambda: [U.to_dev(U.rand_values(rng, n, F32), F32) for _ in range(world)]
     for op in ("avg", "min", "max", "product"):
         t = mk()
-        assert launches(lambda: H.allreduce_replay(t, op, BUTTERFLY, wire_bf16=True, mode=FUSED)) == 3, op
+        assert launches(lambda: H.allreduce_replay(t, op, BUTTERFLY, wire_bf16=True, mode=FUSED)) == (2 if op == "avg" else 3), op
     t = mk()
-    assert launches(lambda: H.allreduce_replay(t, "sum", BUTTERFLY, mode=FUSED)) == 1 + 1   # 6 copies of 400 KB: one launch
+    assert launches(lambda: H.allreduce_replay(t, "sum", BUTTERFLY, mode=FUSED)) == 1
+    t = mk()
+    assert launches(lambda: H.allreduce_replay(t, "max", BUTTERFLY, mode=FUSED)) == 1 + 1   # 6 copies of 400 KB: one launch
+    five = [U.to_dev(U.rand_values(rng, n, F32), F32) for _ in range(5)]
+    assert launches(lambda: H.allreduce_replay(five, "sum", RING, mode=FUSED)) == 1 + 1
+    assert launches(lambda: H.allreduce_replay(five, "avg", RING, wire_bf16=True, mode=FUSED)) == 3
     t = mk()
     stepwise = launches(lambda: H.allreduce_replay(t, "avg", BUTTERFLY, wire_bf16=True, mode=STEPWISE))
     assert stepwise >= 3 + 2 * 3 * 2 + 3 + 3       # encodes, (copy + reduce) per peer and rank, scales, ..., decodes
     groups = [[U.to_dev(U.rand_values(rng, 5000 + 7 * i, F32), F32) for _ in range(world)] for i in range(200)]
-    assert launches(lambda: H.allreduce_replay_many(groups, "sum", TREE)) == 2
+    assert launches(lambda: H.allreduce_replay_many(groups, "sum", TREE)) == 1
     wide = [U.to_dev(U.rand_values(rng, n, F32), F32) for _ in range(16)]     # 16 ranks: folds of 8, 8 and 2 operands
     assert launches(lambda: H.allreduce_replay(wide, "avg", RING, wire_bf16=True, mode=FUSED)) == 1 + 3 + 1
     small = [U.to_dev(U.rand_values(rng, 1000, F32), F32) for _ in range(20)]  # tree of 20: blocks 8 + 8 + 4, then 3
