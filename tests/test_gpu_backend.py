@@ -2,6 +2,7 @@
 tests/test_smoke.py) and N ranks as N threads of one process sharing the GPU,
 checked bit for bit against the oracle's replay of the reference."""
 import datetime
+import gc
 import os
 import threading
 
@@ -115,6 +116,8 @@ def test_distributed_data_parallel_over_the_backend_world_one(CX):
                 opt.step()
         assert torch.equal(plain.weight, wrapped.module.weight)
     finally:
+        wrapped = opt_b = model = opt = None   # a DDP module sits in reference cycles: collected here, while its group exists
+        gc.collect()
         dist.destroy_process_group()
 
 
