@@ -628,7 +628,7 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
 
     # whole allreduce of the bucket for all 3 virtual ranks: fused vs the reference's launch sequence
     ws = H.Workspace(q, 3 * (numel * 2 + 256) + 3 * (2 * ((numel + 2) // 3) * 2 + 256))
-    for mode, name in ((L.REPLAY_FUSED, "fused"), (L.REPLAY_STEPWISE, "stepwise")):
+    for mode, name in ((L.REPLAY_DIRECT, "direct"), (L.REPLAY_FUSED, "fused"), (L.REPLAY_STEPWISE, "stepwise")):
         def rep(i, mode=mode):
             H.allreduce_replay(tensors[i % sets], "avg", L.ALGO_BUTTERFLY, wire_bf16=True, mode=mode,
                                queue=q, workspace=ws, sync=False)
@@ -642,18 +642,23 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
             rep(i)
         ms = q.timer_end()
         out[f"c2_allreduce_{name}_us_per_bucket"] = round(ms / steps * 1e3, 1)
-    # the fused schedule again, its launches recorded into a graph (no host launch cost between them)
+    # the fused schedules again, their launches recorded into a graph (no host launch cost between
+    # them): FUSED = encode + a fold over bf16 copies (the shape across GPUs), DIRECT = ONE fold that
+    # reads the three fp32 tensors and stores the result into all three (ranks sharing one GPU:
+    # 12 B read + 12 B written per element)
     import ctypes as C
-    reps = []
-    for s in range(sets):
-        r = L.Replay()
-        r.world, r.algo, r.op, r.dtype = world, L.ALGO_BUTTERFLY, L.AVG, L.F32
-        r.wire_bf16, r.mode, r.acc, r.reserved, r.numel = 1, L.REPLAY_FUSED, L.ACC_STEP, 0, numel
-        ptrs = (C.c_void_p * world)(*[t.data_ptr() for t in tensors[s]])
-        r.tensors, r.workspace, r.workspace_bytes = ptrs, ws.ptr, ws.nbytes
-        reps.append((r, ptrs))
-    ms, _ = measure(lambda i: L.check(L.lib().mcclx_allreduce_replay(q.handle, C.byref(reps[i % sets][0]))), steps, warm)
-    out["c2_allreduce_fused_in_graph_us_per_bucket"] = round(ms / steps * 1e3, 1)
+    for mode, name in ((L.REPLAY_FUSED, "fused"), (L.REPLAY_DIRECT, "direct")):
+        reps = []
+        for s in range(sets):
+            r = L.Replay()
+            r.world, r.algo, r.op, r.dtype = world, L.ALGO_BUTTERFLY, L.AVG, L.F32
+            r.wire_bf16, r.mode, r.acc, r.reserved, r.numel = 1, mode, L.ACC_STEP, 0, numel
+            ptrs = (C.c_void_p * world)(*[t.data_ptr() for t in tensors[s]])
+            r.tensors, r.workspace, r.workspace_bytes = ptrs, ws.ptr, ws.nbytes
+            reps.append((r, ptrs))
+        ms, _ = measure(lambda i: L.check(L.lib().mcclx_allreduce_replay(q.handle, C.byref(reps[i % sets][0]))), steps, warm)
+        out[f"c2_allreduce_{name}_in_graph_us_per_bucket"] = round(ms / steps * 1e3, 1)
+    out["c2_allreduce_direct_in_graph_GBps"] = round(gbs(world * numel * 8, ms / steps), 1)
     ws.free()
 
     # C1: ring, 2 ranks, 1 Mi fp32, SUM: one k=2 fold per chunk

@@ -32,8 +32,9 @@ extern "C" {
 
 #define MCCLX_API __attribute__((visibility("default")))
 /* 2: mcclx_plan.flags (was a reserved field that had to be 0), mcclx_fold_batched_noalloc,
- *    mcclx_probe_stream.  Layouts of version 1 callers stay valid. */
-#define MCCLX_ABI_VERSION 2
+ *    mcclx_probe_stream.  Layouts of version 1 callers stay valid.
+ * 3: MCCLX_IO_ALL_F32, MCCLX_REPLAY_DIRECT.  Layouts unchanged. */
+#define MCCLX_ABI_VERSION 3
 #define MCCLX_MAX_INPUTS 8 /* inputs one launch folds; wider worlds chain launches */
 
 /* ---- codes ---------------------------------------------------------------- */
@@ -65,7 +66,11 @@ enum {
     MCCLX_IO_PURE = 0,          /* every input and the output are W                     */
     MCCLX_IO_OUT_F32 = 1,       /* W = bf16: inputs bf16, output fp32 (decode on store) */
     MCCLX_IO_OWN_FIRST_F32 = 2, /* W = bf16: in[0] fp32 (encoded in registers), out fp32 */
-    MCCLX_IO_OWN_LAST_F32 = 3   /* W = bf16: in[k-1] fp32, out fp32 (ring order)        */
+    MCCLX_IO_OWN_LAST_F32 = 3,  /* W = bf16: in[k-1] fp32, out fp32 (ring order)        */
+    MCCLX_IO_ALL_F32 = 4        /* W = bf16: every input fp32 (each encoded in registers,
+                                   the cast of ProcessGroupMCCL.cpp:131-132), out fp32: ranks
+                                   that share one GPU read each other's tensors where they
+                                   lie, and no wire copy is ever written                    */
 };
 
 enum {
@@ -313,7 +318,14 @@ MCCLX_API int mcclx_select_algo(const char* env_algo, int64_t tree_below, uint64
 
 enum {
     MCCLX_REPLAY_STEPWISE = 0, /* the reference's launches one by one (binary reduce per received chunk) */
-    MCCLX_REPLAY_FUSED = 1     /* one multi-input fold per owned chunk, peers read in place */
+    MCCLX_REPLAY_FUSED = 1,    /* one multi-input fold per owned chunk, peers read in place */
+    MCCLX_REPLAY_DIRECT = 2    /* FUSED, and with the wire codec on a sum of up to MCCLX_MAX_INPUTS
+                                  ranks the fold reads every rank's fp32 tensor where it lies and
+                                  encodes it in registers (MCCLX_IO_ALL_F32): no rank writes a bf16
+                                  copy, there is no encode launch.  For ranks that share one GPU,
+                                  where the wire is HBM and an fp32 read costs less than writing
+                                  and re-reading a bf16 copy; across GPUs FUSED keeps the link
+                                  traffic at 2 bytes per element.  Elsewhere the same as FUSED.  */
 };
 
 typedef struct {
@@ -323,7 +335,7 @@ typedef struct {
     int32_t dtype;      /* dtype of the rank tensors                                   */
     int32_t wire_bf16;  /* MCCL_WIRE_DTYPE=bf16 (only acts on fp32 tensors)            */
     int32_t mode;       /* MCCLX_REPLAY_*                                              */
-    int32_t acc;        /* MCCLX_ACC_* (FUSED only)                                    */
+    int32_t acc;        /* MCCLX_ACC_* (FUSED and DIRECT only)                         */
     int32_t reserved;
     uint64_t numel;
     void* const* tensors;  /* world device pointers; reduced in place                  */
@@ -332,13 +344,15 @@ typedef struct {
 } mcclx_replay;
 
 /* Scratch a replay needs: the recv scratch of ProcessGroupMCCL.cpp:152-162 per
- * virtual rank plus, with the wire codec, one bf16 copy per rank. */
+ * virtual rank plus, with the wire codec, one bf16 copy per rank.  0 for a
+ * DIRECT replay whose fold also hands the result to every rank (a sum of up to
+ * four ranks): `workspace` may then be NULL. */
 MCCLX_API uint64_t mcclx_replay_workspace_bytes(const mcclx_replay* r);
 
 /* Single-process replay of allreduce_ring / _tree / _butterfly
  * (AllreduceAlgos.cpp:52-206) for `world` virtual ranks whose tensors all live
  * on this GPU: every send/recv becomes a device copy (STEPWISE) or a direct
- * read of the peer's chunk (FUSED).  Both modes produce bit-identical tensors. */
+ * read of the peer's chunk (FUSED, DIRECT).  All modes produce bit-identical tensors. */
 MCCLX_API int mcclx_allreduce_replay(mcclx_ctx* ctx, const mcclx_replay* r);
 
 /* The same for a list of tensors, as ProcessGroupMCCL::allreduce takes one

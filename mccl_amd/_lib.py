@@ -21,11 +21,11 @@ OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_STATE, ERR_NOMEM = 0, -1, -2, -3,
 F32, F16, BF16 = 0, 1, 2
 SUM, AVG, PRODUCT, MIN, MAX = 0, 1, 2, 3, 4
 SCALE_NONE, SCALE_VIEW, SCALE_TENSOR = 0, 1, 2
-IO_PURE, IO_OUT_F32, IO_OWN_FIRST_F32, IO_OWN_LAST_F32 = 0, 1, 2, 3
+IO_PURE, IO_OUT_F32, IO_OWN_FIRST_F32, IO_OWN_LAST_F32, IO_ALL_F32 = 0, 1, 2, 3, 4
 TOPO_FOLD, TOPO_BINOMIAL = 0, 1
 ACC_STEP, ACC_F32 = 0, 1
 ALGO_RING, ALGO_TREE, ALGO_BUTTERFLY = 0, 1, 2
-REPLAY_STEPWISE, REPLAY_FUSED = 0, 1
+REPLAY_STEPWISE, REPLAY_FUSED, REPLAY_DIRECT = 0, 1, 2
 PLAN_ACC_IS_SRC = 1
 
 

@@ -20,7 +20,7 @@ OBJ_DIR = os.path.join(ROOT, "build", "mcclx")
 LIB_PATH = os.path.join(HERE, "libmcclx.so")
 
 SOURCES = ["fold_kernels.hip", "copy_kernel.hip", "static_table.hip", "mcclx_api.cpp", "mcclx_sched.cpp"]
-FOLD_PARTS = 6  # fold_kernels.hip is compiled once per part (-DMCCLX_PART=n), in parallel
+FOLD_PARTS = 7  # fold_kernels.hip is compiled once per part (-DMCCLX_PART=n), in parallel
 HEADERS = ["fold_launch.h", "mcclx_internal.h", os.path.join(ROOT, "include", "mcclx.h")]
 
 # -ffp-contract=off / -fno-fast-math: IEEE fp32 add and mul, no FMA fusion, so

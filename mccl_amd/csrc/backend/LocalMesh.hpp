@@ -49,6 +49,7 @@ struct Contribution {
     void* work = nullptr;          // the rank's completion object, when the leader (or a later
                                    // launch) settles it instead of the rank itself
     int async = 0;                 // allreduce: event-based completion asked for (ranks must agree)
+    int direct = 1;                // allreduce: read peers' fp32 tensors in place (rank 0's setting is used)
     int transport = 0;             // allreduce: 0 = peers read in place, 1 = pinned host wire, 2 = staged host wire
     std::vector<uint64_t> in_off;  // all-to-all: byte offsets (or sizes) of what goes to each peer
     std::vector<uint64_t> out_off; // all-to-all: byte offsets (or sizes) of what comes from each peer

@@ -614,6 +614,10 @@ bool env_async_allreduce() {
     const char* e = std::getenv("MCCL_ALLREDUCE_ASYNC");  // re-read on every call, like the other knobs
     return e && e[0] == '1';
 }
+bool env_direct() {
+    const char* e = std::getenv("MCCL_DIRECT");
+    return !(e && e[0] == '0');
+}
 // MCCL_WIRE: unset / "device" = peers' chunks are read where they lie in HBM;
 // "host" = through pinned, device-mapped host memory; "staged" = through the staging pool.
 int env_transport() {
@@ -675,6 +679,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
     c.kind = K_ALLREDUCE;
     c.stream = my_stream();
     c.async = async ? 1 : 0;
+    c.direct = env_direct() ? 1 : 0;
     c.transport = transport;
     c.work = work.get();
     flush_engine_();
@@ -757,14 +762,14 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
             rp.op = all[0].op;
             rp.dtype = all[0].dtype[i];
             rp.wire_bf16 = all[0].wire_bf16;
-            rp.mode = MCCLX_REPLAY_FUSED;
+            // all ranks of this build share one GPU: over the wire codec the fold reads the
+            // peers' fp32 tensors where they lie (MCCL_DIRECT=0: through bf16 copies, the
+            // shape the same schedule has across GPUs)
+            rp.mode = all[0].direct ? MCCLX_REPLAY_DIRECT : MCCLX_REPLAY_FUSED;
             rp.acc = MCCLX_ACC_STEP;
             rp.numel = all[0].numel[i];
             rp.tensors = ptrs[i].data();
-            // size for the stepwise fallback too (a tree of more than 64 ranks)
-            mcclx_replay st = rp;
-            st.mode = MCCLX_REPLAY_STEPWISE;
-            need[i] = (std::max(mcclx_replay_workspace_bytes(&rp), mcclx_replay_workspace_bytes(&st)) + 255) / 256 * 256;
+            need[i] = (mcclx_replay_workspace_bytes(&rp) + 255) / 256 * 256;
             offset[i] = total;
             total += need[i];
         }

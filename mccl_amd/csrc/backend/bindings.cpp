@@ -244,7 +244,7 @@ std::vector<double> allreduce_rate_probe(int world, int64_t numel, int buckets, 
 //             the right neighbour, receive from the left; AllreduceAlgos.cpp:62-69) with
 //             messages of growing length; every rank checks what it received byte by byte.
 //  "kept":    the same with send_kept: the payload is not copied, and the receiver's copy
-//             must release the sender's hold on the buffer.
+//             must release the transport's hold on the buffer.
 //  "short":   the receiver expects more bytes than were sent.
 //  "silent":  nobody sends; recv must time out and leave the mesh usable for a later exchange.
 std::vector<std::string> peer_wire_probe(const std::string& mode, int world, int rounds, int timeout_ms) {
@@ -284,7 +284,7 @@ std::vector<std::string> peer_wire_probe(const std::string& mode, int world, int
                     return;
                 }
                 long held = 0;
-                std::shared_ptr<std::vector<uint8_t>> previous;
+                std::vector<std::shared_ptr<std::vector<uint8_t>>> sent;
                 for (int i = 0; i < rounds; ++i) {
                     const size_t len = static_cast<size_t>(i) * 1000 + (i == 0 ? 0 : 17);  // the first message is empty
                     auto buf = std::make_shared<std::vector<uint8_t>>(len);
@@ -298,12 +298,15 @@ std::vector<std::string> peer_wire_probe(const std::string& mode, int world, int
                     peer.recv(left, got.data(), len);
                     for (size_t k = 0; k < len; ++k)
                         if (got[k] != pattern(left, i, k)) throw mccl::MCCLError("wrong byte in message " + std::to_string(i));
-                    if (mode == "kept") {
-                        // our message is released once the right neighbour has taken it; it
-                        // takes it before it can send us round i+1, so check one round late
-                        if (previous && previous.use_count() != 1) ++held;
-                        previous = buf;
-                    }
+                    if (mode == "kept") sent.push_back(buf);
+                }
+                if (mode == "kept") {
+                    // a message is released when its receiver's recv returns: once every rank
+                    // has finished its rounds nobody but the sender may hold one
+                    mesh->rendezvous(r, mccl::Contribution{}, std::chrono::milliseconds(20000),
+                                     [](const std::vector<mccl::Contribution>&) {});
+                    for (auto& b : sent)
+                        if (b.use_count() != 1) ++held;
                 }
                 out[static_cast<size_t>(r)] = "ok:" + std::to_string(held);
             } catch (const std::exception& e) {

@@ -74,14 +74,18 @@ constexpr int kBlock = MCCLX_TUNE_BLOCK;  // threads per block of folds that mix
 #ifndef MCCLX_TUNE_F32_BLOCK
 #define MCCLX_TUNE_F32_BLOCK 64
 #endif
+#ifndef MCCLX_TUNE_ALLF32_BLOCK
+#define MCCLX_TUNE_ALLF32_BLOCK 64  // every operand fp32, encoded in registers (MCCLX_IO_ALL_F32)
+#endif
 // Block size by plan, each measured on MI355X.  Folds whose streams all have one
 // element size -- all 16-bit (16 bytes per lane and operand) or all fp32 -- run
 // one-wavefront blocks with one packet per lane: a 512-lane block keeps its wave
 // slots until the last of its loads is back, 64-lane blocks turn them over eight
 // times as often (two to eight 16-bit operands of 512 MiB: +5...9 %, fp32
-// operands: +3...4 %; launches of a few MB are level).  Folds that mix an fp32
-// stream with 16-bit peers (the wire-codec folds) are fastest at 512, and so are
-// one-operand passes.
+// operands: +3...4 %; launches of a few MB are level; fp32 operands encoded in
+// registers, MCCLX_IO_ALL_F32: +7 % on 256 MiB tensors, +1.5 % on 25 MiB ones).
+// Folds that mix an fp32 stream with 16-bit peers (the wire-codec folds) are
+// fastest at 512, and so are one-operand passes.
 constexpr int kWideBlock = MCCLX_TUNE_WIDE_BLOCK;
 constexpr int kWideU = MCCLX_TUNE_WIDE_U;
 
@@ -222,7 +226,7 @@ struct Cfg {
     // elements per packet: 4 as soon as one stream (operand or output) is fp32
     static constexpr int E = (W == MCCLX_F32 || IO != MCCLX_IO_PURE) ? 4 : 8;
     __host__ __device__ static constexpr bool in_is_f32(int k) {
-        return W == MCCLX_F32 || (IO == MCCLX_IO_OWN_FIRST_F32 && k == 0) ||
+        return W == MCCLX_F32 || IO == MCCLX_IO_ALL_F32 || (IO == MCCLX_IO_OWN_FIRST_F32 && k == 0) ||
                (IO == MCCLX_IO_OWN_LAST_F32 && k == K - 1);
     }
     // Packets per lane per iteration.  Measured on MI355X (one block per tile,
@@ -236,7 +240,8 @@ struct Cfg {
                              : ((E == 8 || (K == 1 && IO != MCCLX_IO_PURE)) ? 2 : 1);
     static constexpr bool kDecode = (K == 1 && IO == MCCLX_IO_OUT_F32);  // bf16 -> fp32 cast: +3 % at 64
     static constexpr int BLOCK = kWide ? kWideBlock
-                                 : ((W == MCCLX_F32 && K >= 2) || kDecode) ? MCCLX_TUNE_F32_BLOCK : kBlock;  // threads per block
+                                 : ((W == MCCLX_F32 && K >= 2) || kDecode) ? MCCLX_TUNE_F32_BLOCK
+                                 : (IO == MCCLX_IO_ALL_F32 && K >= 2) ? MCCLX_TUNE_ALLF32_BLOCK : kBlock;  // threads per block
 };
 
 typedef u32x4 RawPack;  // one packet of one operand: 16 B, or 8 B in .xy (16-bit operand, E = 4)
@@ -812,7 +817,9 @@ static bool key_is_wide(const PlanKey& key) { return key_pack_elems(key) == 8 &&
 
 int plan_block(const PlanKey& key) {
     const bool decode = key.k == 1 && key.io == MCCLX_IO_OUT_F32;
-    return key_is_wide(key) ? kWideBlock : ((key.dtype == MCCLX_F32 && key.k >= 2) || decode ? MCCLX_TUNE_F32_BLOCK : kBlock);
+    if (key_is_wide(key)) return kWideBlock;
+    if ((key.dtype == MCCLX_F32 && key.k >= 2) || decode) return MCCLX_TUNE_F32_BLOCK;
+    return (key.io == MCCLX_IO_ALL_F32 && key.k >= 2) ? MCCLX_TUNE_ALLF32_BLOCK : kBlock;
 }
 
 bool fan_plan_ok(const PlanKey& key) {
@@ -868,12 +875,14 @@ int plan_unroll(const PlanKey& key) {
             MCCLX_TOPO_CASES(MCCLX_BF16, MCCLX_IO_OWN_FIRST_F32, MCCLX_SUM, ACC)                   \
         case MCCLX_IO_OWN_LAST_F32:                                                                \
             MCCLX_K_CASES(MCCLX_BF16, MCCLX_IO_OWN_LAST_F32, MCCLX_TOPO_FOLD, MCCLX_SUM, ACC)      \
+        case MCCLX_IO_ALL_F32: return launch_part_sum_bf16_all_f32(st, key, lp);                   \
         default: return hipErrorInvalidValue;                                                      \
     }
 
 hipError_t launch_part_sum_f32_f16(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
 hipError_t launch_part_sum_bf16_step(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
 hipError_t launch_part_sum_bf16_f32acc(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
+hipError_t launch_part_sum_bf16_all_f32(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
 hipError_t launch_part_ops_f32(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
 hipError_t launch_part_ops_f16(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
 hipError_t launch_part_ops_bf16(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
@@ -886,6 +895,8 @@ hipError_t launch_fold(hipStream_t st, const PlanKey& key, const LaunchParams& l
             return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_OWN_FIRST_F32, 3, 0, 0, 0>>(st, lp);
         if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_OWN_FIRST_F32 && key.k == 1)
             return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_OWN_FIRST_F32, 1, 0, 0, 0>>(st, lp);
+        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_ALL_F32 && key.k == 3)
+            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_ALL_F32, 3, 0, 0, 0>>(st, lp);
         if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_OWN_LAST_F32 && key.k == 4)
             return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_OWN_LAST_F32, 4, 0, 0, 0>>(st, lp);
         if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_PURE && key.k == 8)
@@ -966,6 +977,16 @@ hipError_t launch_part_ops_f16(hipStream_t st, const PlanKey& key, const LaunchP
 #if MCCLX_HAS_PART(5)
 hipError_t launch_part_ops_bf16(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
     MCCLX_OTHER_OPS(MCCLX_BF16)
+}
+#endif
+
+#if MCCLX_HAS_PART(6)
+// every operand fp32, encoded in registers (MCCLX_IO_ALL_F32)
+hipError_t launch_part_sum_bf16_all_f32(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
+    if (key.acc == MCCLX_ACC_STEP) {
+        MCCLX_TOPO_CASES(MCCLX_BF16, MCCLX_IO_ALL_F32, MCCLX_SUM, MCCLX_ACC_STEP)
+    }
+    MCCLX_TOPO_CASES(MCCLX_BF16, MCCLX_IO_ALL_F32, MCCLX_SUM, MCCLX_ACC_F32)
 }
 #endif
 

@@ -207,7 +207,7 @@ int check_plan(const mcclx_plan* p, mcclx::PlanKey* key, float* scale_f, int* ha
         return fail(MCCLX_ERR_INVALID, "plan.k=%d outside 1..%d", p->k, MCCLX_MAX_INPUTS);
     int op;
     if (int rc = normalize_op(p->op, &op)) return rc;
-    if (p->io < MCCLX_IO_PURE || p->io > MCCLX_IO_OWN_LAST_F32)
+    if (p->io < MCCLX_IO_PURE || p->io > MCCLX_IO_ALL_F32)
         return fail(MCCLX_ERR_INVALID, "plan.io=%d unknown", p->io);
     if (p->io != MCCLX_IO_PURE && p->dtype != MCCLX_BF16)
         return fail(MCCLX_ERR_UNSUPPORTED, "fp32 operands/outputs need the bf16 wire dtype");
@@ -245,7 +245,7 @@ int check_plan(const mcclx_plan* p, mcclx::PlanKey* key, float* scale_f, int* ha
 }
 
 bool in_is_f32(const mcclx::PlanKey& k, int i) {
-    return k.dtype == MCCLX_F32 || (k.io == MCCLX_IO_OWN_FIRST_F32 && i == 0) ||
+    return k.dtype == MCCLX_F32 || k.io == MCCLX_IO_ALL_F32 || (k.io == MCCLX_IO_OWN_FIRST_F32 && i == 0) ||
            (k.io == MCCLX_IO_OWN_LAST_F32 && i == k.k - 1);
 }
 

@@ -65,11 +65,16 @@ struct Layout {
     uint64_t total;
 };
 
+int fan_of(const mcclx_replay* r);
+bool direct_applies(const mcclx_replay* r);
+
 Layout layout_of(const mcclx_replay* r) {
     Layout L;
     L.wire = r->wire_bf16 && r->dtype == MCCLX_F32;  // ProcessGroupMCCL.cpp:131
     L.wdtype = L.wire ? MCCLX_BF16 : r->dtype;
-    L.wire_stride = L.wire ? align_up(r->numel * 2) : 0;
+    // a DIRECT fold that also hands the result to every rank needs no bf16 copy at all
+    const bool no_copies = direct_applies(r) && fan_of(r) > 0;
+    L.wire_stride = (L.wire && !no_copies) ? align_up(r->numel * 2) : 0;
     L.scratch_off = L.wire_stride * (uint64_t)r->world;
     bool need_scratch = r->mode == MCCLX_REPLAY_STEPWISE || r->world > MCCLX_MAX_INPUTS;
     L.scratch_stride =
@@ -247,6 +252,13 @@ bool all_on_wire(const mcclx_replay* r) {
     return (r->op != MCCLX_SUM && r->op != MCCLX_AVG) || r->world > MCCLX_MAX_INPUTS;
 }
 
+// DIRECT: a sum over the wire codec whose operands fit one fold reads every
+// rank's fp32 tensor itself and encodes it in registers -- the bits of
+// `t.to(at::kBFloat16)` (ProcessGroupMCCL.cpp:131-132) without the bf16 copy.
+bool direct_applies(const mcclx_replay* r) {
+    return r->mode == MCCLX_REPLAY_DIRECT && r->wire_bf16 && r->dtype == MCCLX_F32 && !all_on_wire(r);
+}
+
 // A fold takes MCCLX_MAX_INPUTS operands.  A wider world is folded by a chain
 // of passes over same-dtype buffers: the first takes 8 operands, every later
 // one the partial result plus up to 7 more, in the schedule's own order -- a
@@ -303,7 +315,9 @@ void plan_phases(const mcclx_replay* r, const Layout& L, Phases& ph) {
     if (r->algo == MCCLX_ALGO_TREE) fold.topo = MCCLX_TOPO_BINOMIAL;
     ph.fan = fan_of(r);
     if (ph.fan) fold.flags |= MCCLX_PLAN_FANOUT(ph.fan);
-    if (L.wire && !all_on_wire(r)) {  // the owner's operand is read as fp32 and encoded in registers
+    if (direct_applies(r)) {          // every operand is read as fp32 and encoded in registers
+        fold.io = MCCLX_IO_ALL_F32;
+    } else if (L.wire && !all_on_wire(r)) {  // the owner's operand is read as fp32 and encoded in registers
         if (r->algo == MCCLX_ALGO_TREE)
             fold.io = MCCLX_IO_OWN_FIRST_F32;
         else
@@ -328,10 +342,11 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
     memset(&z, 0, sizeof z);
 
     const bool bf16_only = L.wire && all_on_wire(r);
+    const bool direct = direct_applies(r);  // peers' fp32 tensors are the operands: nothing is encoded
     if (r->algo == MCCLX_ALGO_TREE) {
         // allreduce_tree: rank 0 ends with the binomial combination of all
         // tensors (AllreduceAlgos.cpp:100-114), everyone else receives a copy.
-        if (L.wire)
+        if (L.wire && !direct)
             for (int q = bf16_only ? 0 : 1; q < N; ++q) {  // ranks 1.. encode: their tensors travel
                 mcclx_seg s = z;
                 s.wire_out = wire_of(q);
@@ -378,7 +393,7 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
         } else {
             s.out = r->tensors[0];
             s.in[0] = r->tensors[0];
-            for (int q = 1; q < N; ++q) s.in[q] = L.wire ? wire_of(q) : r->tensors[q];
+            for (int q = 1; q < N; ++q) s.in[q] = (L.wire && !direct) ? wire_of(q) : r->tensors[q];
             if (ph.fan) {  // rank 0's fold hands the result to ranks 1..N-1 itself
                 for (int q = 1; q < N; ++q) s.in[N + q - 1] = r->tensors[q];
             } else if (L.wire) {
@@ -413,7 +428,7 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
         return (j - 1 < chunk) ? j - 1 : j;  // ascending peers, skipping the owner
     };
 
-    if (L.wire)  // every rank encodes what it sends: all chunks except the one it owns
+    if (L.wire && !direct)  // every rank encodes what it sends: all chunks except the one it owns
         for (int q = 0; q < N; ++q)
             for (int ch = 0; ch < N; ++ch) {
                 if ((owner_of(ch) == q && !bf16_only) || c[ch].elem_count == 0) continue;
@@ -431,7 +446,7 @@ void collect_fused(const mcclx_replay* r, const Layout& L, Phases& ph) {
         std::vector<const void*> ops((size_t)N);
         for (int j = 0; j < N; ++j) {
             int q = order_of(ch, j);
-            if (L.wire && (q != o || bf16_only))
+            if (L.wire && !direct && (q != o || bf16_only))
                 ops[(size_t)j] = at(wire_of(q), (uint64_t)c[ch].elem_start * es);
             else
                 ops[(size_t)j] = at(r->tensors[q], (uint64_t)c[ch].elem_start * ts);
@@ -512,7 +527,7 @@ int check_replay(mcclx_ctx* ctx, const mcclx_replay* r, bool* fused, bool* nothi
     if (!ctx || !r || !r->tensors) return bad("replay: null argument");
     if (r->world < 1 || r->reserved != 0) return bad("replay: bad world");
     if (r->algo < MCCLX_ALGO_RING || r->algo > MCCLX_ALGO_BUTTERFLY) return bad("replay: bad algo");
-    if (r->mode != MCCLX_REPLAY_STEPWISE && r->mode != MCCLX_REPLAY_FUSED) return bad("replay: bad mode");
+    if (r->mode < MCCLX_REPLAY_STEPWISE || r->mode > MCCLX_REPLAY_DIRECT) return bad("replay: bad mode");
     if (r->op < MCCLX_SUM || r->op > MCCLX_MAX) {
         // surfaces "Unsupported ReduceOp: n" through the kernel layer
         return mcclx_reduce(ctx, r->tensors[0], r->tensors[0], r->dtype, 0, r->op);
@@ -529,7 +544,7 @@ int check_replay(mcclx_ctx* ctx, const mcclx_replay* r, bool* fused, bool* nothi
     Layout L = layout_of(r);
     if (L.total > 0 && (!r->workspace || r->workspace_bytes < L.total)) return bad("workspace too small");
     // the tree is fused as a tree of 8-rank trees: up to 8 x 8 ranks
-    *fused = r->mode == MCCLX_REPLAY_FUSED &&
+    *fused = r->mode != MCCLX_REPLAY_STEPWISE &&
              (r->algo != MCCLX_ALGO_TREE || r->world <= MCCLX_MAX_INPUTS * MCCLX_MAX_INPUTS);
     return MCCLX_OK;
 }
@@ -567,7 +582,7 @@ bool overlaps(const std::vector<Range>& a, const std::vector<Range>& b) {
 // Same plan for every phase?
 bool same_plan(const mcclx_replay* a, const mcclx_replay* b) {
     return a->world == b->world && a->algo == b->algo && a->op == b->op && a->dtype == b->dtype &&
-           (a->wire_bf16 != 0) == (b->wire_bf16 != 0) && a->acc == b->acc;
+           (a->wire_bf16 != 0) == (b->wire_bf16 != 0) && a->acc == b->acc && a->mode == b->mode;
 }
 
 }  // namespace
@@ -605,7 +620,15 @@ int mcclx_select_algo(const char* env_algo, int64_t tree_below, uint64_t wire_nb
 
 uint64_t mcclx_replay_workspace_bytes(const mcclx_replay* r) {
     if (!r || r->world < 1) return 0;
-    return layout_of(r).total;
+    uint64_t need = layout_of(r).total;
+    if (r->mode != MCCLX_REPLAY_STEPWISE && r->algo == MCCLX_ALGO_TREE &&
+        r->world > MCCLX_MAX_INPUTS * MCCLX_MAX_INPUTS) {  // runs the stepwise schedule (check_replay)
+        mcclx_replay s = *r;
+        s.mode = MCCLX_REPLAY_STEPWISE;
+        const uint64_t step = layout_of(&s).total;
+        need = step > need ? step : need;
+    }
+    return need;
 }
 
 int mcclx_allreduce_replay(mcclx_ctx* ctx, const mcclx_replay* r) {
@@ -662,7 +685,7 @@ int mcclx_reduce_scatter_shares(mcclx_ctx* ctx, int world, void* const* outs,
     if (world == 1) return mcclx_copy(ctx, outs[0], share(0, 0), cb);  // ProcessGroupMCCL.cpp:333-337
     // MIN / MAX / PRODUCT and fp16 round after every step by definition
     bool step_only = (op != MCCLX_SUM && op != MCCLX_AVG) || dtype == MCCLX_F16;
-    if (mode != MCCLX_REPLAY_FUSED) {
+    if (mode == MCCLX_REPLAY_STEPWISE) {
         for (int r = 0; r < world; ++r) {  // :357, :378-386
             TRY(mcclx_copy(ctx, outs[r], share(r, r), cb));
             for (int p = 0; p < world; ++p)

@@ -34,7 +34,7 @@ def test_header_symbols_are_all_exported_and_bound(L):
         assert hasattr(raw, n), f"{n} declared in mcclx.h but not exported"
         assert n in L.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(L.SIGNATURES) == names
-    assert L.lib().mcclx_abi_version() == 2
+    assert L.lib().mcclx_abi_version() == 3
 
 
 def test_struct_layouts_match_header(L):

@@ -335,15 +335,20 @@ def test_divergent_argument_error_fails_every_rank_at_once(CX):
         assert ok == [6.0] * 5
 
 
-@pytest.mark.parametrize("queues", [1, 2])
-def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypatch, queues):
+@pytest.mark.parametrize("queues,direct", [(1, True), (2, True), (2, False)])
+def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypatch, queues, direct):
     """MCCL_ALLREDUCE_ASYNC=1: allreduce returns a pending Work, wait() orders the caller's
     stream after the reduce queue without blocking the host, the Future settles from the
     completion ticket, and buckets issued while two earlier launches are still in flight go
     out together (one launch per phase for all of them).  With two queues (the default) the
     buckets alternate between them, up to two launches in flight on each.  Results are the oracle's,
-    bit for bit."""
+    bit for bit.  By default the fold reads the ranks' fp32 tensors itself (one kernel per launch);
+    MCCL_DIRECT=0 goes through bf16 copies (an encode in front of the fold)."""
     monkeypatch.setenv("MCCL_ALLREDUCE_ASYNC", "1")
+    if direct:
+        monkeypatch.delenv("MCCL_DIRECT", raising=False)
+    else:
+        monkeypatch.setenv("MCCL_DIRECT", "0")
     monkeypatch.setenv("MCCL_ASYNC_QUEUES", str(queues))
     monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "butterfly")
     monkeypatch.setenv("MCCL_WIRE_DTYPE", "bf16")
@@ -394,7 +399,8 @@ def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypat
     # together, 3 launches; two queues -- two at once on either queue, behind them buckets 4 and
     # 6 together and bucket 5, 6 launches.  A rank thread that is held up may split a group.
     assert (3 if queues == 1 else 6) <= l1 - l0 < len(sizes), "buckets were coalesced"
-    assert k1 - k0 == 2 * (l1 - l0), "a launch of several buckets is encode + fold (which also hands out the result), once"
+    assert k1 - k0 == (1 if direct else 2) * (l1 - l0), \
+        "a launch of several buckets is one fold that also hands out the result (behind one encode without MCCL_DIRECT), once"
     assert all(all(out[r][2]) for r in range(world)), "a Work was complete when allreduce returned"
 
 

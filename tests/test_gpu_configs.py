@@ -45,7 +45,7 @@ def test_c2_butterfly_bucket_full(env):
     rc, algo = orc.pg_allreduce(want, F32, AVG, wire_bf16=True, env_algo="butterfly", threads=8)
     assert rc == 0 and algo == BUTTERFLY
     assert np.array_equal(want[0], want[1]) and np.array_equal(want[1], want[2])
-    for mode in (STEPWISE, FUSED):
+    for mode in (STEPWISE, FUSED, L.REPLAY_DIRECT):
         d = [U.to_dev(x, F32) for x in xs]
         H.allreduce_replay(d, "avg", L.ALGO_BUTTERFLY, wire_bf16=True, mode=mode)
         for r in range(3):
@@ -83,6 +83,11 @@ def test_c3_ring_110m_ragged_hbm_and_pinned_host(env):
         assert torch.equal(fused[r].view(torch.int32), step[r].view(torch.int32)), f"rank {r}: fused != stepwise"
         assert torch.equal(fused[r].view(torch.int32), fused[0].view(torch.int32)), "ranks differ"
     del step
+    direct = [t.clone() for t in base]     # one launch: the fold reads the four fp32 tensors where they lie
+    H.allreduce_replay(direct, "sum", L.ALGO_RING, wire_bf16=True, mode=L.REPLAY_DIRECT)
+    for r in range(world):
+        assert torch.equal(fused[r].view(torch.int32), direct[r].view(torch.int32)), f"rank {r}: fused != direct"
+    del direct
     # oracle on windows: chunk c folds x_c, x_{c+1}, ..., owner last (AllreduceAlgos.cpp:62-75)
     for lo, hi in _windows(chunks, numel):
         host = [t[lo:hi].cpu().numpy() for t in base]

@@ -98,7 +98,7 @@ def test_fold_other_ops_and_fp16(K, U, k, dtype, binomial):
 
 
 @pytest.mark.parametrize("k", range(1, 9))
-@pytest.mark.parametrize("io", ["out_f32", "own_first", "own_last"])
+@pytest.mark.parametrize("io", ["out_f32", "own_first", "own_last", "all_f32"])
 @pytest.mark.parametrize("binomial", [False, True])
 def test_fold_wire_modes(K, U, k, io, binomial):
     """fp32 tensors with the bf16 wire codec in one pass == encode, k-1 binary
@@ -108,10 +108,14 @@ def test_fold_wire_modes(K, U, k, io, binomial):
     rng = np.random.default_rng(100 * k + len(io))
     n = 30011
     own = U.rand_values(rng, n, F32, scale=1e-3, specials=True)
-    peers = [U.rand_values(rng, n, BF16, scale=1e-3, specials=True) for _ in range(k - (io != "out_f32"))]
+    if io == "all_f32":  # every operand an fp32 tensor, each encoded in registers
+        peers32 = [U.rand_values(rng, n, F32, scale=1e-3, specials=True) for _ in range(k - 1)]
+        peers = [orc.encode_bf16(p) for p in peers32]
+    else:
+        peers = [U.rand_values(rng, n, BF16, scale=1e-3, specials=True) for _ in range(k - (io != "out_f32"))]
     if io == "out_f32":
         ops = peers
-    elif io == "own_first":
+    elif io in ("own_first", "all_f32"):
         ops = [orc.encode_bf16(own)] + peers
     else:
         ops = peers + [orc.encode_bf16(own)]
@@ -122,7 +126,10 @@ def test_fold_wire_modes(K, U, k, io, binomial):
         down = U.to_dev(own, F32)
         out = torch.empty(n, dtype=torch.float32, device="cuda")
         wire = torch.empty(n, dtype=torch.bfloat16, device="cuda")
-        if io == "out_f32":
+        if io == "all_f32":
+            dp = [U.to_dev(p, F32) for p in peers32]
+            ptrs, code = [down.data_ptr()] + [t.data_ptr() for t in dp], L().IO_ALL_F32
+        elif io == "out_f32":
             ptrs, code = [t.data_ptr() for t in dp], L().IO_OUT_F32
         elif io == "own_first":
             ptrs, code = [down.data_ptr()] + [t.data_ptr() for t in dp], L().IO_OWN_FIRST_F32
@@ -434,7 +441,7 @@ def test_scale_after_a_fold_keeps_the_sign_of_zero(K, U, dtype, op):
                 U.assert_same_bits(out, v[0], dtype, f"dtype {dtype} op {op} k {k} scale {scale}")
 
 
-@pytest.mark.parametrize("kind", ["f32", "bf16", "f16", "own_first", "own_last"])
+@pytest.mark.parametrize("kind", ["f32", "bf16", "f16", "own_first", "own_last", "all_f32"])
 def test_fan_out_writes_the_result_to_every_destination(K, U, kind):
     """MCCLX_PLAN_FANOUT(n): what `out` receives also goes to in[k .. k+n-1] -- the owner of a
     chunk handing the reduced values to every other rank (AllreduceAlgos.cpp:77-86,185-200)
@@ -442,7 +449,8 @@ def test_fan_out_writes_the_result_to_every_destination(K, U, kind):
     destinations, a destination that is one of the operands, by-value and table launches."""
     rng = np.random.default_rng(len(kind) * 7)
     dtype = {"f32": F32, "bf16": BF16, "f16": F16}.get(kind, BF16)
-    io = {"own_first": L().IO_OWN_FIRST_F32, "own_last": L().IO_OWN_LAST_F32}.get(kind, L().IO_PURE)
+    io = {"own_first": L().IO_OWN_FIRST_F32, "own_last": L().IO_OWN_LAST_F32,
+          "all_f32": L().IO_ALL_F32}.get(kind, L().IO_PURE)
     odt = F32 if (dtype == F32 or io != L().IO_PURE) else dtype
     es = {F32: 4, F16: 2, BF16: 2}
     for k in range(2, 8):
@@ -454,7 +462,8 @@ def test_fan_out_writes_the_result_to_every_destination(K, U, kind):
                     n = int(rng.integers(1, 30000 if nseg < 10 else 3000))
                     ins, ptrs, dev = [], [], []
                     for j in range(k):
-                        f32_in = dtype == F32 or (kind == "own_first" and j == 0) or (kind == "own_last" and j == k - 1)
+                        f32_in = (dtype == F32 or kind == "all_f32" or (kind == "own_first" and j == 0) or
+                                  (kind == "own_last" and j == k - 1))
                         dt = F32 if f32_in else dtype
                         off = int(rng.integers(0, 5))
                         a = U.rand_values(rng, n + off + 4, dt, scale=1e-2, specials=(dt != F16))

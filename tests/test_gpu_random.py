@@ -163,6 +163,8 @@ def allreduce_case(case, rng, H, U):
     dtype, wire = [(F32, False), (BF16, False), (F16, False), (F32, True)][int(rng.integers(0, 4))]
     op = int(rng.choice([SUM, AVG, MIN, MAX, PRODUCT]))
     mode = int(rng.integers(0, 2))
+    if mode == 1 and case % 2:   # FUSED, or DIRECT (over the wire codec: the ranks' fp32 tensors read in place)
+        mode = 2
     many = rng.integers(0, 3) == 0
     groups = int(rng.integers(2, 7)) if many else 1
     desc = f"case {case}: allreduce algo {NAMES[algo]} world {world} dtype {dtype} wire {wire} op {op} mode {mode} groups {groups}"
@@ -239,9 +241,15 @@ def collective_mix_case(case, rng, monkeypatch, CX, U):
     for _ in range(int(rng.integers(3, 10))):
         kind = int(rng.choice([0, 0, 0, 1, 2, 3]))
         steps.append((kind, int(rng.integers(0, ntens)), int(rng.integers(0, ntens)), int(rng.choice([SUM, MAX, MIN, AVG]))))
-    desc = f"case {case}: world {world} dtype {dtype} async {asyn} queues {queues} chunk {chunk} steps {steps}"
-    for k in ("MCCL_ALLREDUCE_ALGO", "MCCL_WIRE", "MCCL_ALLREDUCE_ASYNC", "MCCL_WIRE_DTYPE"):
+    wire = dtype == F32 and case % 2 == 1            # the bf16 wire codec on the allreduces ...
+    direct = case % 4 != 3                           # ... whose fold reads the fp32 tensors itself, or bf16 copies
+    desc = f"case {case}: world {world} dtype {dtype} async {asyn} queues {queues} chunk {chunk} wire {wire} direct {direct} steps {steps}"
+    for k in ("MCCL_ALLREDUCE_ALGO", "MCCL_WIRE", "MCCL_ALLREDUCE_ASYNC", "MCCL_WIRE_DTYPE", "MCCL_DIRECT"):
         monkeypatch.delenv(k, raising=False)
+    if wire:
+        monkeypatch.setenv("MCCL_WIRE_DTYPE", "bf16")
+    if not direct:
+        monkeypatch.setenv("MCCL_DIRECT", "0")
     monkeypatch.setenv("MCCL_ASYNC_QUEUES", queues)
     if asyn:
         monkeypatch.setenv("MCCL_ALLREDUCE_ASYNC", "1")
@@ -272,10 +280,10 @@ def collective_mix_case(case, rng, monkeypatch, CX, U):
     WS = [[small[r][t].copy() for r in range(world)] for t in range(ntens)]
     for kind, i, j, op in steps:
         if kind == 0:
-            assert orc.pg_allreduce(WB[i], dtype, op)[0] == 0
+            assert orc.pg_allreduce(WB[i], dtype, op, wire_bf16=wire)[0] == 0
         elif kind == 1:
-            assert orc.pg_allreduce(WS[j], dtype, op)[0] == 0
-            assert orc.pg_allreduce(WB[i], dtype, op)[0] == 0
+            assert orc.pg_allreduce(WS[j], dtype, op, wire_bf16=wire)[0] == 0
+            assert orc.pg_allreduce(WB[i], dtype, op, wire_bf16=wire)[0] == 0
         elif kind == 2:
             assert orc.reduce_scatter(WS[j], WB[i], dtype, op) == 0
         else:

@@ -34,7 +34,7 @@ def U():
     return gpu_util
 
 
-STEPWISE, FUSED = 0, 1
+STEPWISE, FUSED, DIRECT = 0, 1, 2
 
 
 def run_case(H, U, algo, world, dtype, op, wire, mode, numel, seed, specials=False):
@@ -56,7 +56,7 @@ def run_case(H, U, algo, world, dtype, op, wire, mode, numel, seed, specials=Fal
 
 @pytest.mark.parametrize("algo", [RING, TREE, BUTTERFLY])
 @pytest.mark.parametrize("world", [2, 3, 4, 5, 8])
-@pytest.mark.parametrize("mode", [STEPWISE, FUSED])
+@pytest.mark.parametrize("mode", [STEPWISE, FUSED, DIRECT])
 @pytest.mark.parametrize("dtype,wire", [(F32, False), (BF16, False), (F32, True)])
 def test_allreduce_sum_avg(H, U, algo, world, mode, dtype, wire):
     for op in (SUM, AVG):
@@ -67,7 +67,7 @@ def test_allreduce_sum_avg(H, U, algo, world, mode, dtype, wire):
 
 @pytest.mark.parametrize("algo", [RING, TREE, BUTTERFLY])
 @pytest.mark.parametrize("op", [PRODUCT, MIN, MAX])
-@pytest.mark.parametrize("mode", [STEPWISE, FUSED])
+@pytest.mark.parametrize("mode", [STEPWISE, FUSED, DIRECT])
 def test_allreduce_other_ops_and_fp16(H, U, algo, op, mode):
     for world in (2, 3, 4):
         for dtype, wire in ((F32, False), (BF16, False), (F16, False), (F32, True)):
@@ -387,7 +387,15 @@ def test_launch_counts_of_the_fused_schedules(H, K, U):
     assert launches(lambda: H.allreduce_replay(t, "sum", BUTTERFLY, mode=FUSED)) == 1
     t = mk()
     assert launches(lambda: H.allreduce_replay(t, "max", BUTTERFLY, mode=FUSED)) == 1 + 1   # 6 copies of 400 KB: one launch
+    # DIRECT: the fold reads the ranks' fp32 tensors itself -- the whole wire allreduce of up to
+    # four ranks is one launch, of five to eight a fold and the casts on arrival
+    for algo in (RING, TREE, BUTTERFLY):
+        t = mk()
+        assert launches(lambda: H.allreduce_replay(t, "avg", algo, wire_bf16=True, mode=DIRECT)) == 1
+    t = mk()
+    assert launches(lambda: H.allreduce_replay(t, "max", BUTTERFLY, wire_bf16=True, mode=DIRECT)) == 3
     five = [U.to_dev(U.rand_values(rng, n, F32), F32) for _ in range(5)]
+    assert launches(lambda: H.allreduce_replay(five, "avg", RING, wire_bf16=True, mode=DIRECT)) == 2
     assert launches(lambda: H.allreduce_replay(five, "sum", RING, mode=FUSED)) == 1 + 1
     assert launches(lambda: H.allreduce_replay(five, "avg", RING, wire_bf16=True, mode=FUSED)) == 3
     t = mk()
