@@ -625,6 +625,21 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
                [K.make_seg(0, wires[s][r].data_ptr(), [tensors[s][r].data_ptr()], numel) for r in range(world)])
     ms, _ = measure(enc, steps, warm)
     out["c2_encode_GBps"] = round(gbs(world * numel * 6, ms / steps), 1)
+    # its ceilings: the plain copy kernel over the same footprint (118 MB per launch, cold) and the
+    # same encode on a tensor large enough for the fixed cost of a launch not to matter (64 Mi elements)
+    half = world * numel * 3
+    pool = torch.randint(0, 256, (8 * half,), dtype=torch.uint8, device="cuda")
+    ms, _ = measure(lambda i: q.copy(pool.data_ptr() + (2 * (i % 4) + 1) * half, pool.data_ptr() + 2 * (i % 4) * half, half),
+                    steps, warm)
+    out["c2_encode_footprint_plain_copy_GBps"] = round(gbs(2 * half, ms / steps), 1)
+    del pool
+    nbig = 64 << 20
+    src = [torch.randn(nbig, device="cuda") * 1e-3 for _ in range(2)]
+    dst = [torch.empty(nbig, dtype=torch.bfloat16, device="cuda") for _ in range(2)]
+    ms, _ = measure(lambda i: q.fold(K.make_plan(L.BF16, 1, io=L.IO_OWN_FIRST_F32),
+                                     [K.make_seg(0, dst[i % 2].data_ptr(), [src[i % 2].data_ptr()], nbig)]), 10, 2)
+    out["encode_64Mi_elements_GBps"] = round(gbs(nbig * 6, ms / 10), 1)
+    del src, dst
 
     # whole allreduce of the bucket for all 3 virtual ranks: fused vs the reference's launch sequence
     ws = H.Workspace(q, 3 * (numel * 2 + 256) + 3 * (2 * ((numel + 2) // 3) * 2 + 256))

@@ -100,13 +100,13 @@ struct ProcessGroupMCCL::Shared {
     // with one submission, which removes the host's launch gaps between them.
     // The key is everything the launches depend on; MCCL_GRAPH_CACHE=0 turns it off.
     struct GraphKey {
-        int world, algo, op, dtype, wire;
+        int world, algo, op, dtype, wire, mode;
         uint64_t numel;
         void* workspace;
         std::vector<void*> tensors;
         bool operator<(const GraphKey& o) const {
-            return std::tie(world, algo, op, dtype, wire, numel, workspace, tensors) <
-                   std::tie(o.world, o.algo, o.op, o.dtype, o.wire, o.numel, o.workspace, o.tensors);
+            return std::tie(world, algo, op, dtype, wire, mode, numel, workspace, tensors) <
+                   std::tie(o.world, o.algo, o.op, o.dtype, o.wire, o.mode, o.numel, o.workspace, o.tensors);
         }
     };
     struct GraphEntry {
@@ -389,7 +389,7 @@ struct ProcessGroupMCCL::Shared {
             check_rc(mcclx_allreduce_replay(ctx, &rp));
             return;
         }
-        GraphKey key{rp.world, rp.algo, rp.op, rp.dtype, rp.wire_bf16, rp.numel, rp.workspace,
+        GraphKey key{rp.world, rp.algo, rp.op, rp.dtype, rp.wire_bf16, rp.mode, rp.numel, rp.workspace,
                      std::vector<void*>(rp.tensors, rp.tensors + rp.world)};
         GraphEntry& e = graphs[key];
         e.last_use = ++use_clock;
