@@ -112,7 +112,12 @@ struct ProcessGroupMCCL::Shared {
     struct GraphEntry {
         mcclx_graph* graph = nullptr;
         uint64_t seen = 0, last_use = 0;
+        uint64_t launches = 0;  // kernel launches of its first, eager issue
     };
+    // Replaying a recorded graph costs the host about 22 us whatever it holds, an eager
+    // launch 3.5 us: only an allreduce of this many launches or more is recorded
+    // (MCCL_GRAPH_MIN_LAUNCHES; a sum of up to eight ranks is one or two launches).
+    uint64_t graph_min_launches = 6;
     static constexpr size_t kMaxGraphs = 256;
     std::map<GraphKey, GraphEntry> graphs;
     uint64_t use_clock = 0;
@@ -170,6 +175,7 @@ struct ProcessGroupMCCL::Shared {
     Shared() {
         const char* e = std::getenv("MCCL_GRAPH_CACHE");
         graphs_enabled = !(e && e[0] == '0');
+        if (const char* m = std::getenv("MCCL_GRAPH_MIN_LAUNCHES")) graph_min_launches = std::strtoull(m, nullptr, 10);
         const char* q = std::getenv("MCCL_ASYNC_QUEUES");
         if (q && q[0] == '1') queues = 1;
     }
@@ -382,8 +388,8 @@ struct ProcessGroupMCCL::Shared {
         return reinterpret_cast<void*>((p + 255) / 256 * 256);
     }
 
-    // One allreduce of the group: replayed from its graph when there is one,
-    // recorded on its second occurrence, issued launch by launch otherwise.
+    // One allreduce of the group: issued launch by launch and counted the first time;
+    // one of many launches is recorded on its second occurrence and replayed from then on.
     void allreduce(const mcclx_replay& rp) {
         if (!graphs_enabled) {
             check_rc(mcclx_allreduce_replay(ctx, &rp));
@@ -394,7 +400,14 @@ struct ProcessGroupMCCL::Shared {
         GraphEntry& e = graphs[key];
         e.last_use = ++use_clock;
         ++e.seen;
-        if (!e.graph && e.seen >= 2) {
+        if (e.seen == 1) {  // issued eagerly, and counted
+            const uint64_t before = mcclx_launch_count(ctx);
+            check_rc(mcclx_allreduce_replay(ctx, &rp));
+            e.launches = mcclx_launch_count(ctx) - before;
+            if (graphs.size() > kMaxGraphs) evict();
+            return;
+        }
+        if (!e.graph && e.launches >= graph_min_launches) {
             check_rc(mcclx_graph_begin(ctx));
             int rc = mcclx_allreduce_replay(ctx, &rp);
             std::string why = rc == MCCLX_OK ? "" : mcclx_last_error();

@@ -817,6 +817,7 @@ def test_repeated_allreduce_is_replayed_from_a_graph_and_stays_bit_exact(CX, U, 
     else:
         monkeypatch.delenv("MCCL_WIRE_DTYPE", raising=False)
     monkeypatch.delenv("MCCL_GRAPH_CACHE", raising=False)
+    monkeypatch.setenv("MCCL_GRAPH_MIN_LAUNCHES", "1")   # by default only allreduces of six launches or more are recorded
     rng = np.random.default_rng(77)
     rounds = 8
     data = [[U.rand_values(rng, n, F32, scale=1e-2, specials=(i == 3)) for _ in range(world)] for i in range(rounds)]
