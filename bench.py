@@ -546,9 +546,13 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
 
     # NOT the headline: consecutive buckets on TWO reduce queues (two contexts, two streams), so that
     # one launch's ramp-up fills the other's drain and the gap between dependent launches is hidden.
-    # Out-of-place results as in the headline; wall clock around both graphs, best of 5.
+    # Out-of-place results as in the headline; wall clock around both graphs, best of 5.  Launches
+    # that overlap do not have the memory system to themselves: the hold form (reads, then writes)
+    # is switched off on both queues, as the process group does when it runs two queues.
     q2 = K.ReduceQueue(0)
     try:
+        q.set_hold(False)
+        q2.set_hold(False)
         per_q = max(50, steps // 2)
         graphs = []
         for qi, qq in enumerate((q, q2)):
@@ -572,6 +576,7 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
         out["c2_fold_overlapped_on_two_queues_us_per_bucket"] = round(best / (2 * per_q) * 1e6, 2)
         out["c2_fold_overlapped_on_two_queues_GBps"] = round(numel * 12 / (best / (2 * per_q)) / 1e9, 1)
     finally:
+        q.set_hold(True)
         del q2
 
     # C2 with the peers' bf16 chunks left where a NIC or a host transport puts them: pinned host

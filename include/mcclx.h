@@ -33,7 +33,8 @@ extern "C" {
 #define MCCLX_API __attribute__((visibility("default")))
 /* 2: mcclx_plan.flags (was a reserved field that had to be 0), mcclx_fold_batched_noalloc,
  *    mcclx_probe_stream.  Layouts of version 1 callers stay valid.
- * 3: MCCLX_IO_ALL_F32, MCCLX_REPLAY_DIRECT.  Layouts unchanged. */
+ * 3: MCCLX_IO_ALL_F32, MCCLX_REPLAY_DIRECT, mcclx_set_hold, mcclx_hold_launch_count.
+ *    Layouts unchanged. */
 #define MCCLX_ABI_VERSION 3
 #define MCCLX_MAX_INPUTS 8 /* inputs one launch folds; wider worlds chain launches */
 
@@ -110,6 +111,23 @@ MCCLX_API int mcclx_device_cus(mcclx_ctx* ctx);
 /* Diagnostic: kernel launches this context has issued so far (recorded ones
  * count when they are recorded, not when a graph replays them). */
 MCCLX_API uint64_t mcclx_launch_count(mcclx_ctx* ctx);
+
+/* The hold form of a fold launch (no counterpart in the reference; results are
+ * the same bits).  A launch that mixes reads and writes streams about 10 %
+ * slower on this part than one that only reads or only writes.  A by-value
+ * fold launch (up to 32 segments) of two to four operands that reads at least
+ * 12 MiB and is small enough for one generation of blocks to cover it -- a
+ * 25 MiB gradient bucket is -- therefore issues all its loads first, holds its
+ * results in registers and stores them only when its reads are through: the
+ * host passes, from the bytes the launch reads, the time before which no lane
+ * stores.  That model assumes the launch has the memory system to itself: a
+ * queue whose launches run next to other work on the GPU (a second reduce
+ * queue) does better without it.  enabled = 0 switches the form off for this
+ * context, 1 on again; MCCLX_HOLD=0 in the environment switches it off for
+ * every context made afterwards. */
+MCCLX_API int mcclx_set_hold(mcclx_ctx* ctx, int enabled);
+/* Diagnostic: launches of this context that took the hold form. */
+MCCLX_API uint64_t mcclx_hold_launch_count(mcclx_ctx* ctx);
 
 /* ---- the reference's four kernel entry points, one to one ------------------- */
 

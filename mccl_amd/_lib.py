@@ -74,6 +74,8 @@ SIGNATURES = {
     "mcclx_queue_stream": (_vp, [_vp]),
     "mcclx_device_cus": (_i, [_vp]),
     "mcclx_launch_count": (_u64, [_vp]),
+    "mcclx_hold_launch_count": (_u64, [_vp]),
+    "mcclx_set_hold": (_i, [_vp, _i]),
     "mcclx_reduce": (_i, [_vp, _vp, _vp, _i, _u64, _i]),
     "mcclx_scale": (_i, [_vp, _vp, _i, _u64, _d, _i]),
     "mcclx_accumulate_scale": (_i, [_vp, _vp, _vp, _i, _u64, _d]),

@@ -633,6 +633,170 @@ __global__ void __launch_bounds__(C::BLOCK) fold_few_wide_kernel(FewArgs a) { fo
 template <class C>
 __global__ void __launch_bounds__(C::BLOCK) fold_few_fan_kernel(FewArgs a) { fold_few_body<C, true>(a); }
 
+#if MCCLX_TUNE_TIMELINE
+// Where the next by-value launches put their records: a caller-provided device
+// buffer cut into `slots` regions of `per_slot` records, used round robin.
+static TimelineRecord* g_tl_buf = nullptr;
+static uint64_t g_tl_slots = 0, g_tl_per_slot = 0, g_tl_next = 0;
+static TimelineRecord* timeline_next(uint64_t blocks) {
+    if (!g_tl_buf || blocks > g_tl_per_slot) return nullptr;
+    return g_tl_buf + (g_tl_next++ % g_tl_slots) * g_tl_per_slot;
+}
+extern "C" MCCLX_API void mcclx_tune_timeline(void* device_buf, uint64_t slots, uint64_t records_per_slot) {
+    g_tl_buf = static_cast<TimelineRecord*>(device_buf);
+    g_tl_slots = slots;
+    g_tl_per_slot = records_per_slot;
+    g_tl_next = 0;
+}
+#endif
+
+// ------------------------------------------------------ reads, then writes
+//
+// A launch that mixes its reads and writes streams about 10 % slower on this
+// part than one that only reads or only writes (the memory bus pays for every
+// change of direction).  A launch small enough for ONE generation of blocks to
+// cover it can keep the two apart: every lane issues the loads of all its T
+// packets at once, folds them as they arrive, keeps the T results in registers
+// and stores them only when the launch's reads are through.  "Through" is a
+// matter of time, not of a barrier: the host knows how many bytes the launch
+// reads and passes the moment (in ticks of the 100 MHz wall clock, counted from
+// the block's own start) before which no lane stores.  A gate that is too late
+// costs its excess, one that is too early lets writes into the reads again --
+// results do not depend on it.  C2 (78.6 MB per launch): 14.1 -> 12.9 us.
+//
+// What one generation holds is set by the vector registers (every packet in
+// flight occupies them until it is stored): the launch takes the first of
+// T = 4 or 5 packets per lane in 512-lane blocks, or 4 in 256-lane blocks,
+// whose one generation covers the longest segment -- C2-shaped folds of up to
+// 32 MiB per rank, the all-fp32 fold of a 25 MiB bucket.
+template <class C, int T, int kHoldBlock, bool FAN>
+__global__ void __launch_bounds__(kHoldBlock) fold_few_hold_kernel(FewArgs a, uint32_t gate) {
+    const uint64_t t_start = wall_clock64();
+    SegArgs s = a.seg[blockIdx.y];
+    float scale = a.scale;
+    int32_t has_scale = a.has_scale;
+    uint32_t grid = gridDim.x;
+    fetch_together<FAN ? MCCLX_MAX_INPUTS : C::K>(s, scale, has_scale, grid);
+    int32_t fan = 0;
+    if constexpr (FAN) fan = a.fan;
+    const uint32_t head = head_elems<C>(s);
+    const uint64_t P = (s.count - head) / C::E;
+    const bool has_out = s.out != nullptr, has_wire = s.wire_out != nullptr;
+    const SegArgs t = advanced<C, FAN>(s, head);
+    // packet u of lane l is packet u * L + l of the segment: consecutive lanes, consecutive packets
+    const uint32_t L = grid * kHoldBlock;
+    const uint32_t lane = blockIdx.x * kHoldBlock + threadIdx.x;
+    // Packet indices are worked out again for the arithmetic and for the stores (behind a
+    // barrier the compiler cannot see through) instead of being kept in registers across
+    // the wait: registers decide how many packets one generation holds.
+    RawPack raw[C::K][T];
+    {
+#pragma unroll
+        for (int u = 0; u < T; ++u) {
+            const uint32_t p = (uint32_t)u * L + lane;
+            if (p < P) {
+                uint32_t one[1] = {p};
+                RawPack col[C::K][1];
+                load_all<C, 0, 1>(t, one, col);
+#pragma unroll
+                for (int k = 0; k < C::K; ++k) raw[k][u] = col[k][0];
+            }
+        }
+    }
+    float res[T][C::E];
+    uint32_t lane2 = lane;
+    asm volatile("" : "+v"(lane2));
+#pragma unroll
+    for (int u = 0; u < T; ++u)
+        if ((uint32_t)u * L + lane2 < P) {
+            RawPack col[C::K];
+#pragma unroll
+            for (int k = 0; k < C::K; ++k) col[k] = raw[k][u];
+            combine<C>(col, res[u]);
+            finish_pack<C>(res[u], scale, has_scale != 0);
+        }
+#if MCCLX_TUNE_TIMELINE
+    const uint64_t t_args = wall_clock64();  // here: this block has its data
+#endif
+    // the clock only moves forward, so every wave leaves this loop
+    while (wall_clock64() - t_start < gate) __builtin_amdgcn_s_sleep(8);
+    uint32_t lane3 = lane2;
+    asm volatile("" : "+v"(lane3));
+#pragma unroll
+    for (int u = 0; u < T; ++u) {
+        const uint32_t p = (uint32_t)u * L + lane3;
+        if (p < P) store_pack<C, FAN>(t, has_out, has_wire, p, res[u], fan);
+    }
+    if (blockIdx.x == 0) {  // the elements in front of and behind the packet grid
+        if (threadIdx.x < head) fold_elem<C, FAN>(s, threadIdx.x, scale, has_scale != 0, fan);
+        const uint64_t i = head + P * C::E + threadIdx.x;
+        if (i < s.count) fold_elem<C, FAN>(s, i, scale, has_scale != 0, fan);
+    }
+#if MCCLX_TUNE_TIMELINE
+    if (a.timeline && threadIdx.x == 0) {
+        TimelineRecord r;
+        r.t_start = t_start;
+        r.t_args = t_args;
+        r.t_end = wall_clock64();
+        r.hw_id = __builtin_amdgcn_s_getreg((31 << 11) | 4);
+        r.xcc_id = __builtin_amdgcn_s_getreg((31 << 11) | 20);
+        a.timeline[(uint64_t)blockIdx.y * gridDim.x + blockIdx.x] = r;
+    }
+#endif
+}
+
+// Plans with a reads-then-writes form: sums of two to four operands in packets of four
+// elements (fp32, or the wire-codec folds with an fp32 stream), rounding after every step.
+template <class C>
+constexpr bool kHoldPlan = C::K >= 2 && C::K <= 4 && C::E == 4 && C::OP == MCCLX_SUM && C::ACC == MCCLX_ACC_STEP &&
+                           C::TOPO == MCCLX_TOPO_FOLD;
+
+// Blocks of one generation: what the device holds at once of this kernel.
+template <class C, int T, int HB, bool FAN>
+static uint32_t hold_capacity(int cus) {
+    static const int per_cu = [] {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fold_few_hold_kernel<C, T, HB, FAN>, HB, 0) != hipSuccess) {
+            (void)hipGetLastError();
+            n = 0;
+        }
+        return n;
+    }();
+    return (uint32_t)(per_cu * cus);
+}
+
+template <class C, int T, int HB, bool FAN>
+static bool hold_launch(hipStream_t st, FewArgs& a, uint64_t packets, uint32_t gate, const LaunchParams& lp) {
+    const uint32_t cap = hold_capacity<C, T, HB, FAN>(lp.cus);
+    if (cap < (uint32_t)a.nseg) return false;
+    const uint32_t hx = cap / (uint32_t)a.nseg;
+    if (packets > (uint64_t)hx * HB * T) return false;
+#if MCCLX_TUNE_TIMELINE
+    a.timeline = timeline_next((uint64_t)hx * (uint64_t)a.nseg);
+#endif
+    fold_few_hold_kernel<C, T, HB, FAN><<<dim3(hx, (uint32_t)a.nseg), dim3(HB), 0, st>>>(a, gate);
+    return true;
+}
+
+// Takes the launch if it reads enough for the separation to pay and one generation covers it.
+template <class C, bool FAN>
+static bool try_hold(hipStream_t st, FewArgs& a, uint64_t maxc, const LaunchParams& lp) {
+    if (!lp.hold_min_read_bytes || lp.cus <= 0) return false;
+    uint64_t read_bytes = 0;
+    for (int i = 0; i < a.nseg; ++i)
+        for (int k = 0; k < C::K; ++k) read_bytes += a.seg[i].count * (C::in_is_f32(k) ? 4 : 2);
+    if (read_bytes < lp.hold_min_read_bytes) return false;
+    uint64_t ticks = lp.hold_latency_ticks + read_bytes / lp.hold_bytes_per_tick;
+    const uint32_t gate = ticks > 100000 ? 100000u : (uint32_t)ticks;  // a millisecond at most
+    const uint64_t packets = (maxc + C::E - 1) / C::E;
+    // 512-lane blocks first (a C2 fold: 13.1 us against 14.3 us in 256-lane blocks); the wider
+    // all-fp32 folds only fit one generation in 256-lane blocks
+    const bool took = hold_launch<C, 4, 512, FAN>(st, a, packets, gate, lp) || hold_launch<C, 5, 512, FAN>(st, a, packets, gate, lp) ||
+                      hold_launch<C, 4, 256, FAN>(st, a, packets, gate, lp);
+    if (took && lp.held) *lp.held = true;
+    return took;
+}
+
 // A value that is the same in every lane, moved to scalar registers.  The
 // compiler cannot always prove it (a quotient comes out of the vector ALU), and
 // a descriptor kept in vector registers costs the kernel a quarter of its
@@ -703,22 +867,6 @@ constexpr bool kFanPlan = C::OP == MCCLX_SUM && C::ACC == MCCLX_ACC_STEP && C::K
 
 // ----------------------------------------------------------------- dispatch
 
-#if MCCLX_TUNE_TIMELINE
-// Where the next by-value launches put their records: a caller-provided device
-// buffer cut into `slots` regions of `per_slot` records, used round robin.
-static TimelineRecord* g_tl_buf = nullptr;
-static uint64_t g_tl_slots = 0, g_tl_per_slot = 0, g_tl_next = 0;
-static TimelineRecord* timeline_next(uint64_t blocks) {
-    if (!g_tl_buf || blocks > g_tl_per_slot) return nullptr;
-    return g_tl_buf + (g_tl_next++ % g_tl_slots) * g_tl_per_slot;
-}
-extern "C" MCCLX_API void mcclx_tune_timeline(void* device_buf, uint64_t slots, uint64_t records_per_slot) {
-    g_tl_buf = static_cast<TimelineRecord*>(device_buf);
-    g_tl_slots = slots;
-    g_tl_per_slot = records_per_slot;
-    g_tl_next = 0;
-}
-#endif
 
 #ifdef MCCLX_TUNE_MINIMAL
 static size_t wide_lds_bytes() {  // tuning: dynamic LDS reserved per block of a wide fold, to cap blocks per CU
@@ -754,6 +902,8 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
 #if MCCLX_TUNE_TIMELINE
                 a.timeline = nullptr;
 #endif
+                if constexpr (kHoldPlan<C>)
+                    if (try_hold<C, true>(st, a, maxc, lp)) return hipGetLastError();
                 fold_few_fan_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(C::BLOCK), 0, st>>>(a);
             }
             return hipGetLastError();
@@ -781,6 +931,8 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
 #if MCCLX_TUNE_TIMELINE
         a.timeline = timeline_next(gx * (uint64_t)a.nseg);
 #endif
+        if constexpr (kHoldPlan<C>)
+            if (try_hold<C, false>(st, a, maxc, lp)) return hipGetLastError();
         if constexpr (kLightPlan<C>)
             fold_few_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(C::BLOCK), 0, st>>>(a);
         else

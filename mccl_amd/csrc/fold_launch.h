@@ -73,6 +73,15 @@ struct LaunchParams {
     const TableArgs* table = nullptr;
     uint32_t max_blocks = 0;           // cap on the grid (persistent sizing)
     int fan = 0;                       // > 0: the fan-out form of the kernel (plans in fan_plan_ok only)
+    // Reads-then-writes form of a by-value launch that one generation of blocks covers:
+    // taken when the launch reads at least hold_min_read_bytes (0 = never); no lane stores
+    // before hold_latency_ticks + read bytes / hold_bytes_per_tick ticks of the 100 MHz
+    // wall clock have passed since its block started.
+    int cus = 0;
+    bool* held = nullptr;              // set when the launch took that form (diagnostic)
+    uint64_t hold_min_read_bytes = 0;
+    uint32_t hold_latency_ticks = 90;
+    uint32_t hold_bytes_per_tick = 76000;
 };
 // Plans that have a fan-out form: sums with per-step rounding, 2..7 operands.
 bool fan_plan_ok(const PlanKey& key);

@@ -75,6 +75,11 @@ struct mcclx_ctx {
     std::atomic<uint64_t> launches{0};  // kernel launches issued (diagnostic)
     uint32_t few_max = mcclx::kFewSegs;  // segments up to which descriptors travel in the kernel arguments
     bool validate = false;
+    // reads-then-writes launches (LaunchParams): least bytes read, and the gate's model
+    uint64_t hold_min_read_bytes = 12ull << 20;
+    uint32_t hold_latency_ticks = 90, hold_bytes_per_tick = 76000;
+    bool hold_enabled = true;
+    std::atomic<uint64_t> hold_launches{0};
     bool batch_active = false;
     std::string batch_label;
     std::mutex mu;
@@ -399,6 +404,12 @@ int launch_by_value(mcclx_ctx* ctx, const mcclx::PlanKey& key, float scale_f, in
     mcclx::LaunchParams lp;
     lp.max_blocks = ctx->max_blocks;
     lp.fan = fan;
+    lp.cus = ctx->cus;
+    bool held = false;
+    lp.held = &held;
+    lp.hold_min_read_bytes = ctx->hold_enabled ? ctx->hold_min_read_bytes : 0;
+    lp.hold_latency_ticks = ctx->hold_latency_ticks;
+    lp.hold_bytes_per_tick = ctx->hold_bytes_per_tick;
     mcclx::FewArgs a;
     memset(&a, 0, sizeof a);
     for (uint32_t s = 0; s < nseg; ++s) memcpy(&a.seg[s], &segs[s], sizeof(mcclx_seg));
@@ -409,6 +420,7 @@ int launch_by_value(mcclx_ctx* ctx, const mcclx::PlanKey& key, float scale_f, in
     hipError_t e = mcclx::launch_fold(ctx->stream, key, lp);
     if (e != hipSuccess) return launch_error(e, key);
     ++ctx->launches;
+    if (held) ++ctx->hold_launches;
     return MCCLX_OK;
 }
 
@@ -521,6 +533,17 @@ int make_ctx(int device, hipStream_t borrowed, bool borrow, mcclx_ctx** out) {
         if (x >= 0 && x <= mcclx::kFewSegs) ctx->few_max = (uint32_t)x;
     }
     if (const char* v = getenv("MCCLX_VALIDATE")) ctx->validate = (v[0] == '1');
+    // MCCLX_HOLD=0 switches the reads-then-writes launches off; the other three are tuning knobs
+    if (const char* v = getenv("MCCLX_HOLD")) ctx->hold_enabled = v[0] != '0';
+    if (const char* v = getenv("MCCLX_HOLD_MIN_BYTES")) {
+        const unsigned long long x = strtoull(v, nullptr, 10);
+        ctx->hold_min_read_bytes = x ? x : 1;
+    }
+    if (const char* v = getenv("MCCLX_HOLD_LATENCY_TICKS")) ctx->hold_latency_ticks = (uint32_t)strtoul(v, nullptr, 10);
+    if (const char* v = getenv("MCCLX_HOLD_BYTES_PER_TICK")) {
+        const unsigned long x = strtoul(v, nullptr, 10);
+        if (x >= 1000 && x <= 1000000) ctx->hold_bytes_per_tick = (uint32_t)x;
+    }
     e = mcclx::static_table_resolve(device, &ctx->static_table);  // `device` is current (guard above)
     if (e != hipSuccess) {
         delete ctx;
@@ -593,6 +616,12 @@ int mcclx_destroy(mcclx_ctx* ctx) {
 void* mcclx_queue_stream(mcclx_ctx* ctx) { return ctx ? (void*)ctx->stream : nullptr; }
 int mcclx_device_cus(mcclx_ctx* ctx) { return ctx ? ctx->cus : 0; }
 uint64_t mcclx_launch_count(mcclx_ctx* ctx) { return ctx ? ctx->launches.load() : 0; }
+uint64_t mcclx_hold_launch_count(mcclx_ctx* ctx) { return ctx ? ctx->hold_launches.load() : 0; }
+int mcclx_set_hold(mcclx_ctx* ctx, int enabled) {
+    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
+    ctx->hold_enabled = enabled != 0;
+    return MCCLX_OK;
+}
 
 int mcclx_fold(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* seg) {
     return fold_impl(ctx, plan, seg, 1);

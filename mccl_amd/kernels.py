@@ -182,6 +182,16 @@ class ReduceQueue:
         """Kernel launches issued on this queue so far (diagnostic)."""
         return int(L.lib().mcclx_launch_count(self.handle))
 
+    def hold_launch_count(self) -> int:
+        """Launches of this queue that took the hold form: reads first, results kept in registers,
+        writes once the reads are through (diagnostic)."""
+        return int(L.lib().mcclx_hold_launch_count(self.handle))
+
+    def set_hold(self, enabled: bool) -> None:
+        """Switch the hold form of fold launches off (a queue whose launches overlap with other
+        work on the GPU) or on again."""
+        L.check(L.lib().mcclx_set_hold(self.handle, int(enabled)))
+
     def copy(self, dst_ptr: int, src_ptr: int, nbytes: int) -> None:
         L.check(L.lib().mcclx_copy(self.handle, C.c_void_p(dst_ptr), C.c_void_p(src_ptr), nbytes))
 
