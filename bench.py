@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 CAL_BYTES = 64 << 20   # size of the calibration copy
 # HBM bytes one C2 fold launch moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by the
 # calibration copy (profiles/c2_fold_hbm_traffic_pmc.txt): 1.004 x the algorithmic bytes.
-C2_MEASURED_TRAFFIC_BYTES = 78_941_759
+C2_MEASURED_TRAFFIC_BYTES = 79_063_009
 
 
 def parse():
@@ -200,7 +200,7 @@ def main():
                    "algorithmic_bytes_per_step": bytes_per_step, "parity_vs_oracle_bit_exact": parity},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": C2_MEASURED_TRAFFIC_BYTES,
-                     "kernel": "fold_few_kernel<bf16, own-first fp32, k=3>", "kernel_us": round(kernel_us, 2)},
+                     "kernel": "fold_few_hold_kernel<bf16, own-first fp32, k=3; 4 packets per lane, 512-lane blocks>", "kernel_us": round(kernel_us, 2)},
     }
     extra = {"warm_GBps": round(gbs(bytes_per_step, warm_dev / args.steps), 1),
              "warm_kernel_us": round(warm_dev / args.steps * 1e3, 2),
@@ -289,13 +289,17 @@ def timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure,
     pr("C2 fused fold -- timeline of one launch from per-block time stamps, MI355X (gfx950)")
     pr("")
     pr("Command: python -m mccl_amd.build --timeline   (here, once)   then on the GPU box:   python bench.py --timeline")
-    pr("Every block of fold_few_kernel<bf16, own-first fp32, k=3> records wall_clock64() (100 MHz, 10 ns ticks) at its first")
-    pr("instruction, once its kernel arguments have arrived, and after its last store was issued. 16 consecutive launches")
-    pr("(3201 blocks of 512 threads each: one per 8 KiB tile of a chunk; cold = rotating 8 copies of the workload,")
-    pr("944 MB + 629 MB of results) are recorded into one HIP graph; figures are means over launches 3..15 of its 4th replay.")
-    pr("All times in microseconds.")
+    pr("Every block of the fold <bf16, own-first fp32, k=3> records wall_clock64() (100 MHz, 10 ns ticks) at its first")
+    pr("instruction, at a second point, and after its last store was issued.  16 consecutive launches (cold = rotating 8")
+    pr("copies of the workload, 944 MB + 629 MB of results) are recorded into one HIP graph; figures are means over")
+    pr("launches 3..15 of its 4th replay.  All times in microseconds.")
+    pr("  hold form  (the default for this launch): 1023 blocks of 512 threads, ONE generation; every lane issues the loads")
+    pr("             of its four packets at once, keeps the results in registers and stores them when the gate opens")
+    pr("             (90 ticks + bytes read / 76,000 per tick after its block started).  Second stamp: the block has its data.")
+    pr("  plain form (mcclx_set_hold(ctx, 0); every launch too large for one generation): 3201 blocks, one per 8 KiB tile of")
+    pr("             a chunk, loads then stores.  Second stamp: the block has its kernel arguments.")
 
-    def capture(seg_fn, label):
+    def capture(seg_fn, label, hold=False):
         buf = torch.zeros(slots * per_slot * rec_words, dtype=torch.int64, device="cuda")
         torch.cuda.synchronize()
         set_tl(buf.data_ptr(), slots, per_slot)
@@ -339,6 +343,23 @@ def timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure,
         pr(f"  span:   first block start -> last block's end       {m['span']:6.2f}")
         pr(f"  gap:    last block's end -> next launch's first     {m['gap']:6.2f}   (store acknowledgements, end-of-kernel release, dispatch of the next)")
         pr(f"  inside the span:")
+        t0, ta, t1, xcc = launches[8]
+        s0 = t0.min()
+        if hold:
+            data = [(np.sort(l[1])[[0, len(l[1]) // 2, -1]] - l[0].min()) * tick for l in launches[2:slots - 1]]
+            d0, d50, d100 = (float(np.mean([d[j] for d in data])) for j in range(3))
+            pr(f"    all {int(m['blocks'])} blocks started after                     {m['last_start']:6.2f}")
+            pr(f"    first / median / last block has its data after    {d0:6.2f} / {d50:.2f} / {d100:.2f}   (the launch's reads are through)")
+            pr(f"    first block past its gate, first store issued     {m['first_end']:6.2f}   (nothing has been written before this)")
+            pr(f"    last store issued (the span)                      {m['span']:6.2f}")
+            pr(f"    spread of the 8 XCDs' finishing times             {m['xcd_spread']:6.2f}")
+            m.update(data_first=d0, data_last=d100)
+            pr(f"  launch 9 of the 16, per microsecond since its first block started:")
+            pr(f"    t       started   have their data   stores issued")
+            for b in range(0, int((t1.max() - s0) * tick) + 1):
+                lo, hi = s0 + b * 100, s0 + (b + 1) * 100
+                pr(f"    {b:2d}-{b + 1:<2d}   {int(((t0 >= lo) & (t0 < hi)).sum()):6d}  {int(((ta >= lo) & (ta < hi)).sum()):10d}  {int(((t1 >= lo) & (t1 < hi)).sum()):14d}")
+            return m
         pr(f"    {4 * cus} blocks (all wave slots) started after        {m['fill']:6.2f}")
         pr(f"    a block waits for its kernel arguments            {m['args']:6.2f}   (mean)")
         pr(f"    first block has its data and ends after           {m['first_end']:6.2f}   (nothing has been written before this)")
@@ -347,8 +368,6 @@ def timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure,
         pr(f"    the last 10 % of block ends take                  {m['last90']:6.2f}   (a tenth of the span would be {0.1 * m['span']:.2f})")
         pr(f"    spread of the 8 XCDs' finishing times             {m['xcd_spread']:6.2f}")
         # one launch in 1 us bins
-        t0, ta, t1, xcc = launches[8]
-        s0 = t0.min()
         pr(f"  launch 9 of the 16, per microsecond since its first block started:")
         pr(f"    t       started   ended   resident   GB/s by block ends")
         per_block = bytes_per_step / len(t0)
@@ -361,13 +380,21 @@ def timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure,
         return m
 
     sets = args.sets
-    cold = capture(lambda i: q.fold(plan, step_segs(i % sets, out_tensors=results[i % sets])), "cold: rotating copies, reads from HBM")
-    warm = capture(lambda i: q.fold(plan, step_segs(0, out_tensors=results[0])), "warm: one copy, resident in the 256 MiB Infinity Cache")
+    cold_fn = lambda i: q.fold(plan, step_segs(i % sets, out_tensors=results[i % sets]))
+    warm_fn = lambda i: q.fold(plan, step_segs(0, out_tensors=results[0]))
+    held = capture(cold_fn, "hold form, cold: rotating copies, reads from HBM", hold=True)
+    capture(warm_fn, "hold form, warm: one copy, resident in the 256 MiB Infinity Cache", hold=True)
+    q.set_hold(False)
+    cold = capture(cold_fn, "plain form, cold")
+    capture(warm_fn, "plain form, warm")
 
-    # the same launch without the stamps, and what bounds it: one-directional streams of the same footprint
+    # the same launches without the stamps, and what bounds them: one-directional streams of the same footprint
     gbs = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
     steps = args.steps
-    ms, _ = measure(lambda i: q.fold(plan, step_segs(i % sets, out_tensors=results[i % sets])), steps, args.warmup)
+    ms, _ = measure(cold_fn, steps, args.warmup)
+    plain_us = ms / steps * 1e3
+    q.set_hold(True)
+    ms, _ = measure(cold_fn, steps, args.warmup)
     fold_us = ms / steps * 1e3
     fp = bytes_per_step
     probe = torch.randint(0, 256, (8 * fp,), dtype=torch.uint8, device="cuda")
@@ -385,7 +412,8 @@ def timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure,
     empty_us = ms / steps * 1e3
     pr("")
     pr(f"[the same launches without stamps, {steps} per graph replay, HIP events around the replay; cold]")
-    pr(f"  C2 fold (52.4 MB read + 26.2 MB written)            {fold_us:6.2f} us per launch = {gbs(fp, fold_us * 1e-3):6.0f} GB/s = {gbs(fp, fold_us * 1e-3) / 80:5.1f} % of 8 TB/s")
+    pr(f"  C2 fold (52.4 MB read + 26.2 MB written), hold form {fold_us:6.2f} us per launch = {gbs(fp, fold_us * 1e-3):6.0f} GB/s = {gbs(fp, fold_us * 1e-3) / 80:5.1f} % of 8 TB/s")
+    pr(f"  the same, plain form                                {plain_us:6.2f} us per launch = {gbs(fp, plain_us * 1e-3):6.0f} GB/s = {gbs(fp, plain_us * 1e-3) / 80:5.1f} % of 8 TB/s")
     for name, us, g in lines:
         pr(f"  {name:<50s}  {us:6.2f} us per launch = {g:6.0f} GB/s")
     pr(f"  one-block launch (4 KiB read), back to back         {empty_us:6.2f} us per launch: what two dependent launches cost with no work in them")
@@ -393,9 +421,14 @@ def timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure,
     pr("Reading: a launch's period = gap + span. The gap (last store issued -> first block of the next launch running) is")
     pr("spent on store acknowledgements, the end-of-kernel cache release and the dispatch of the dependent launch; the span")
     pr("opens with one memory latency in which no byte has arrived and closes with a drain in which the queues empty.")
-    pr(f"Cold: {cold['gap']:.2f} gap + {cold['first_end']:.2f} until the first block has data leave "
+    pr(f"Plain form, cold: {cold['gap']:.2f} gap + {cold['first_end']:.2f} until the first block has data leave "
        f"{cold['period'] - cold['gap'] - cold['first_end']:.2f} us in which {fp / 1e6:.1f} MB move: "
-       f"{fp / (cold['period'] - cold['gap'] - cold['first_end']) / 1e3:.0f} GB/s while data flows.")
+       f"{fp / (cold['period'] - cold['gap'] - cold['first_end']) / 1e3:.0f} GB/s while data flows, reads and writes mixed.")
+    rd, wr = fp * 2 / 3, fp / 3
+    pr(f"Hold form, cold: the same {held['gap']:.2f} gap and {held['data_first']:.2f} first round trip; then the reads alone, "
+       f"{rd / 1e6:.1f} MB in {held['data_last'] - held['data_first']:.2f} us = {rd / (held['data_last'] - held['data_first']) / 1e3:.0f} GB/s,")
+    pr(f"then the writes alone, {wr / 1e6:.1f} MB between the first store ({held['first_end']:.2f}) and the last ({held['span']:.2f}) "
+       f"= {wr / (held['span'] - held['first_end']) / 1e3:.0f} GB/s by issue: each direction near what the one-directional launches above reach.")
     print("\n".join(out))
 
 
@@ -527,6 +560,14 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
         out[f"{name}_same_footprint_us"] = round(ms / steps * 1e3, 2)
         out[f"{name}_same_footprint_GBps"] = round(gbs(fp, ms / steps), 1)
     del probe
+
+    # the headline launch in the plain form (one block per tile, loads then stores, reads and writes
+    # mixed on the memory bus) instead of the hold form (all loads, then all stores) it takes by default
+    q.set_hold(False)
+    ms, _ = measure(lambda i: q.fold(plan, step_segs(i % sets, out_tensors=results[i % sets])), steps, warm)
+    q.set_hold(True)
+    out["c2_fold_plain_form_us"] = round(ms / steps * 1e3, 2)
+    out["c2_fold_plain_form_GBps"] = round(gbs(fp, ms / steps), 1)
 
     # the fold as the scheduler issues it: result written in place over the owner's fp32 chunk
     ms, _ = measure(lambda i: q.fold(plan, step_segs(i % sets)), steps, warm)

@@ -928,11 +928,11 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
 #if MCCLX_TUNE_XCD
         gx = (gx + MCCLX_TUNE_XCD - 1) / MCCLX_TUNE_XCD * MCCLX_TUNE_XCD;
 #endif
+        if constexpr (kHoldPlan<C>)
+            if (try_hold<C, false>(st, a, maxc, lp)) return hipGetLastError();
 #if MCCLX_TUNE_TIMELINE
         a.timeline = timeline_next(gx * (uint64_t)a.nseg);
 #endif
-        if constexpr (kHoldPlan<C>)
-            if (try_hold<C, false>(st, a, maxc, lp)) return hipGetLastError();
         if constexpr (kLightPlan<C>)
             fold_few_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(C::BLOCK), 0, st>>>(a);
         else
