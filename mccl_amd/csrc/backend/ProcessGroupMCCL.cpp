@@ -266,9 +266,11 @@ struct ProcessGroupMCCL::Shared {
                 }
                 if (wait_other) check_rc(mcclx_queue_wait_stream(queue(q), mcclx_queue_stream(queue(o))));
             }
-            // launches of two queues overlap on the device, and a launch that does not have the
-            // memory system to itself should not time its stores (mcclx_set_hold)
-            check_rc(mcclx_set_hold(queue(q), alt ? 0 : 1));
+            // an event-based launch runs beside whatever the ranks enqueue next and beside the
+            // other queue's launches, and a launch that does not have the memory system to
+            // itself should not time its stores (mcclx_set_hold; measured beside a stream of
+            // copies: 27.7 us with the hold form, 24.1 us without)
+            check_rc(mcclx_set_hold(queue(q), 0));
             check_rc(mcclx_allreduce_replay_many(queue(q), all.data(), static_cast<uint32_t>(all.size())));
             check_rc(mcclx_event_record(queue(q), &ticket));
         } catch (...) {
@@ -366,7 +368,9 @@ struct ProcessGroupMCCL::Shared {
         }
         main_touched = true;
         if (alt && !flights[1].empty()) check_rc(mcclx_queue_wait_stream(ctx, mcclx_queue_stream(alt)));
-        check_rc(mcclx_set_hold(ctx, 1));  // what follows runs on the main queue alone
+        // what follows waits for the ranks' streams and is drained before anyone goes on:
+        // it has the GPU to itself
+        check_rc(mcclx_set_hold(ctx, 1));
     }
 
     // Host-blocking: nothing of the event-based mode is left on the device.
