@@ -665,10 +665,13 @@ extern "C" MCCLX_API void mcclx_tune_timeline(void* device_buf, uint64_t slots, 
 // results do not depend on it.  C2 (78.6 MB per launch): 14.1 -> 12.9 us.
 //
 // What one generation holds is set by the vector registers (every packet in
-// flight occupies them until it is stored): the launch takes the first of
-// T = 4 or 5 packets per lane in 512-lane blocks, or 4 in 256-lane blocks,
-// whose one generation covers the longest segment -- C2-shaped folds of up to
-// 32 MiB per rank, the all-fp32 fold of a 25 MiB bucket.
+// flight occupies them until it is stored; a packet's result takes the place of
+// its first operand): the launch takes T = 4 or 5 packets per lane, in 512-lane
+// blocks, whichever covers the longest segment in one generation -- C2-shaped
+// folds of up to 40 MiB per rank, the all-fp32 fold of a 25 MiB bucket.  More
+// packets per lane would cover more, but from about 80 MB read on the plain
+// form has caught up (a 40 MiB bucket at T = 7: 21.0 us against 20.7 us); and
+// 256-lane blocks run the C2 fold in 14.3 us where 512-lane blocks take 13.1 us.
 template <class C, int T, int kHoldBlock, bool FAN>
 __global__ void __launch_bounds__(kHoldBlock) fold_few_hold_kernel(FewArgs a, uint32_t gate) {
     const uint64_t t_start = wall_clock64();
@@ -703,7 +706,8 @@ __global__ void __launch_bounds__(kHoldBlock) fold_few_hold_kernel(FewArgs a, ui
             }
         }
     }
-    float res[T][C::E];
+    // a packet's result takes the place of its first operand (kHoldPlan: four elements per packet)
+    static_assert(C::E == 4, "the hold form keeps results where packets of four elements were");
     uint32_t lane2 = lane;
     asm volatile("" : "+v"(lane2));
 #pragma unroll
@@ -712,8 +716,10 @@ __global__ void __launch_bounds__(kHoldBlock) fold_few_hold_kernel(FewArgs a, ui
             RawPack col[C::K];
 #pragma unroll
             for (int k = 0; k < C::K; ++k) col[k] = raw[k][u];
-            combine<C>(col, res[u]);
-            finish_pack<C>(res[u], scale, has_scale != 0);
+            float acc[C::E];
+            combine<C>(col, acc);
+            finish_pack<C>(acc, scale, has_scale != 0);
+            raw[0][u] = u32x4{__float_as_uint(acc[0]), __float_as_uint(acc[1]), __float_as_uint(acc[2]), __float_as_uint(acc[3])};
         }
 #if MCCLX_TUNE_TIMELINE
     const uint64_t t_args = wall_clock64();  // here: this block has its data
@@ -725,7 +731,11 @@ __global__ void __launch_bounds__(kHoldBlock) fold_few_hold_kernel(FewArgs a, ui
 #pragma unroll
     for (int u = 0; u < T; ++u) {
         const uint32_t p = (uint32_t)u * L + lane3;
-        if (p < P) store_pack<C, FAN>(t, has_out, has_wire, p, res[u], fan);
+        if (p < P) {
+            const float y[C::E] = {__uint_as_float(raw[0][u].x), __uint_as_float(raw[0][u].y), __uint_as_float(raw[0][u].z),
+                                   __uint_as_float(raw[0][u].w)};
+            store_pack<C, FAN>(t, has_out, has_wire, p, y, fan);
+        }
     }
     if (blockIdx.x == 0) {  // the elements in front of and behind the packet grid
         if (threadIdx.x < head) fold_elem<C, FAN>(s, threadIdx.x, scale, has_scale != 0, fan);
@@ -789,10 +799,12 @@ static bool try_hold(hipStream_t st, FewArgs& a, uint64_t maxc, const LaunchPara
     uint64_t ticks = lp.hold_latency_ticks + read_bytes / lp.hold_bytes_per_tick;
     const uint32_t gate = ticks > 100000 ? 100000u : (uint32_t)ticks;  // a millisecond at most
     const uint64_t packets = (maxc + C::E - 1) / C::E;
-    // 512-lane blocks first (a C2 fold: 13.1 us against 14.3 us in 256-lane blocks); the wider
-    // all-fp32 folds only fit one generation in 256-lane blocks
-    const bool took = hold_launch<C, 4, 512, FAN>(st, a, packets, gate, lp) || hold_launch<C, 5, 512, FAN>(st, a, packets, gate, lp) ||
-                      hold_launch<C, 4, 256, FAN>(st, a, packets, gate, lp);
+    // the fewest packets per lane whose one generation covers the launch
+#ifdef MCCLX_TUNE_HOLD_256
+    const bool took = hold_launch<C, 4, 256, FAN>(st, a, packets, gate, lp) || hold_launch<C, 5, 256, FAN>(st, a, packets, gate, lp);
+#else
+    const bool took = hold_launch<C, 4, 512, FAN>(st, a, packets, gate, lp) || hold_launch<C, 5, 512, FAN>(st, a, packets, gate, lp);
+#endif
     if (took && lp.held) *lp.held = true;
     return took;
 }

@@ -128,12 +128,13 @@ def test_hold_form_gives_the_oracles_bits(env, queues, kind, k):
     assert plain.hold_launch_count() == 0
 
 
-@pytest.mark.parametrize("kind,k,count", [("own_first", 3, 8_000_000),    # four packets per lane, 512-lane blocks
-                                          ("own_first", 3, 9_500_000),    # five packets per lane
-                                          ("all_f32", 3, 6_553_600),      # 256-lane blocks (or five packets per lane)
+@pytest.mark.parametrize("kind,k,count", [("own_first", 3, 8_000_000),    # four packets per lane
+                                          ("own_first", 3, 9_500_000),    # five
+                                          ("all_f32", 3, 6_553_600),      # the one-launch allreduce of a 25 MiB bucket
+                                          ("own_last", 4, 10_000_000),
                                           ("f32", 2, 7_000_003)])
 def test_hold_form_block_shapes_against_the_plain_form(env, queues, kind, k, count):
-    """Launches near what one generation holds, where the other block shapes take over: the
+    """Launches near what one generation holds, where more packets per lane take over: the
     same bits as the plain form of the same launch."""
     K, L, U, _ = env
     held, plain = queues
@@ -161,7 +162,7 @@ def test_hold_form_block_shapes_against_the_plain_form(env, queues, kind, k, cou
 def test_a_launch_wider_than_one_generation_takes_the_plain_form(env, queues):
     K, L, U, _ = env
     held, _ = queues
-    n = 14_000_000
+    n = 20_000_000
     g = torch.Generator(device="cuda").manual_seed(4)
     own = torch.randn(n, device="cuda", generator=g) * 1e-2
     peers = [(torch.randn(n, device="cuda", generator=g) * 1e-2).to(torch.bfloat16) for _ in range(2)]
