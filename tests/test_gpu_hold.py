@@ -116,7 +116,7 @@ def test_hold_form_gives_the_oracles_bits(env, queues, kind, k):
     rng = np.random.default_rng(1000 + 10 * KINDS.index(kind) + k)
     fans = [0] if kind == "out_f32" else [0, min(2, 8 - k)]
     for fan in fans:
-        for counts in ([1], [7], [4099], [300_007], [33, 70_001, 5], [120_000, 120_001, 119_999]):
+        for counts in ([1], [7], [4099], [300_007], [33, 70_001, 5], [70_001, 0, 9], [120_000, 120_001, 119_999]):
             for in_place in ((False, True) if kind != "out_f32" and fan == 0 else (False,)):
                 plan, segs, checks, keep = build_case(env, rng, kind, k, fan, counts, in_place)
                 before = held.hold_launch_count()
