@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 CAL_BYTES = 64 << 20   # size of the calibration copy
 # HBM bytes one C2 fold launch moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by the
 # calibration copy (profiles/c2_fold_hbm_traffic_pmc.txt): 1.004 x the algorithmic bytes.
-C2_MEASURED_TRAFFIC_BYTES = 79_052_752
+C2_MEASURED_TRAFFIC_BYTES = 79_064_666
 
 
 def parse():
@@ -295,7 +295,7 @@ def timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure,
     pr("launches 3..15 of its 4th replay.  All times in microseconds.")
     pr("  hold form  (the default for this launch): 1023 blocks of 512 threads, ONE generation; every lane issues the loads")
     pr("             of its four packets at once, keeps the results in registers and stores them when the gate opens")
-    pr("             (90 ticks + bytes read / 76,000 per tick after its block started).  Second stamp: the block has its data.")
+    pr("             (40 ticks + bytes read / 71,000 per tick after its block started).  Second stamp: the block has its data.")
     pr("  plain form (mcclx_set_hold(ctx, 0); every launch too large for one generation): 3201 blocks, one per 8 KiB tile of")
     pr("             a chunk, loads then stores.  Second stamp: the block has its kernel arguments.")
 

@@ -116,7 +116,7 @@ MCCLX_API uint64_t mcclx_launch_count(mcclx_ctx* ctx);
  * the same bits).  A launch that mixes reads and writes streams about 10 %
  * slower on this part than one that only reads or only writes.  A by-value
  * fold launch (up to 32 segments) of two to four operands that reads at least
- * 12 MiB and is small enough for one generation of blocks to cover it -- a
+ * 10 MiB (15 MiB with fan-out) and is small enough for one generation of blocks to cover it -- a
  * 25 MiB gradient bucket is -- therefore issues all its loads first, holds its
  * results in registers and stores them only when its reads are through: the
  * host passes, from the bytes the launch reads, the time before which no lane

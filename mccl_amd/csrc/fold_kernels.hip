@@ -795,7 +795,9 @@ static bool try_hold(hipStream_t st, FewArgs& a, uint64_t maxc, const LaunchPara
     uint64_t read_bytes = 0;
     for (int i = 0; i < a.nseg; ++i)
         for (int k = 0; k < C::K; ++k) read_bytes += a.seg[i].count * (C::in_is_f32(k) ? 4 : 2);
-    if (read_bytes < lp.hold_min_read_bytes) return false;
+    // measured break-even: 10 MiB read for a fold with one output, half as much again for one that
+    // writes as much as it reads (fan-out)
+    if (read_bytes < (FAN ? lp.hold_min_read_bytes * 3 / 2 : lp.hold_min_read_bytes)) return false;
     uint64_t ticks = lp.hold_latency_ticks + read_bytes / lp.hold_bytes_per_tick;
     const uint32_t gate = ticks > 100000 ? 100000u : (uint32_t)ticks;  // a millisecond at most
     const uint64_t packets = (maxc + C::E - 1) / C::E;

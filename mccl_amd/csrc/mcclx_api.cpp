@@ -76,8 +76,8 @@ struct mcclx_ctx {
     uint32_t few_max = mcclx::kFewSegs;  // segments up to which descriptors travel in the kernel arguments
     bool validate = false;
     // reads-then-writes launches (LaunchParams): least bytes read, and the gate's model
-    uint64_t hold_min_read_bytes = 12ull << 20;
-    uint32_t hold_latency_ticks = 90, hold_bytes_per_tick = 76000;
+    uint64_t hold_min_read_bytes = 10ull << 20;
+    uint32_t hold_latency_ticks = 40, hold_bytes_per_tick = 71000;
     bool hold_enabled = true;
     std::atomic<uint64_t> hold_launches{0};
     bool batch_active = false;

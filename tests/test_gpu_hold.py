@@ -178,7 +178,7 @@ def test_a_launch_wider_than_one_generation_takes_the_plain_form(env, queues):
 
 
 def test_default_threshold_and_the_switch(env):
-    """By default a launch holds from 12 MiB read on; mcclx_set_hold switches the form off and on."""
+    """By default a launch holds from 10 MiB read on; mcclx_set_hold switches the form off and on."""
     K, L, U, _ = env
     q = queue_with(K)
     try:
