@@ -77,7 +77,8 @@ struct mcclx_ctx {
     bool validate = false;
     // reads-then-writes launches (LaunchParams): least bytes read, and the gate's model
     uint64_t hold_min_read_bytes = 10ull << 20;
-    uint32_t hold_latency_ticks = 40, hold_bytes_per_tick = 71000;
+    uint32_t hold_latency_ticks = 40, hold_bytes_per_tick = 71000;  // in ticks of 100 MHz
+    uint32_t wall_khz = 100000;                                      // the device's wall clock
     bool hold_enabled = true;
     std::atomic<uint64_t> hold_launches{0};
     bool batch_active = false;
@@ -408,8 +409,9 @@ int launch_by_value(mcclx_ctx* ctx, const mcclx::PlanKey& key, float scale_f, in
     bool held = false;
     lp.held = &held;
     lp.hold_min_read_bytes = ctx->hold_enabled ? ctx->hold_min_read_bytes : 0;
-    lp.hold_latency_ticks = ctx->hold_latency_ticks;
-    lp.hold_bytes_per_tick = ctx->hold_bytes_per_tick;
+    lp.hold_latency_ticks = (uint32_t)((uint64_t)ctx->hold_latency_ticks * ctx->wall_khz / 100000);
+    lp.hold_bytes_per_tick = (uint32_t)((uint64_t)ctx->hold_bytes_per_tick * 100000 / ctx->wall_khz);
+    if (lp.hold_bytes_per_tick == 0) lp.hold_bytes_per_tick = 1;
     mcclx::FewArgs a;
     memset(&a, 0, sizeof a);
     for (uint32_t s = 0; s < nseg; ++s) memcpy(&a.seg[s], &segs[s], sizeof(mcclx_seg));
@@ -519,6 +521,14 @@ int make_ctx(int device, hipStream_t borrowed, bool borrow, mcclx_ctx** out) {
         return fail(MCCLX_ERR_HIP, "hipGetDeviceProperties failed: %s", hipGetErrorString(e));
     }
     ctx->cus = prop.multiProcessorCount;
+    // the gate of the hold form is counted in ticks of the device's wall clock: the model's
+    // constants are in ticks of 100 MHz (what gfx950 runs it at) and scaled if the device differs
+    int wall_khz = 0;
+    if (hipDeviceGetAttribute(&wall_khz, hipDeviceAttributeWallClockRate, device) != hipSuccess || wall_khz <= 0) {
+        (void)hipGetLastError();
+        wall_khz = 100000;
+    }
+    ctx->wall_khz = (uint32_t)wall_khz;
     // Grid cap of the table launches.  Default: effectively none -- one block per
     // tile measured fastest (blocks are dispatched in address order; a capped,
     // grid-striding launch loses 5-20 %).  MCCLX_BLOCKS_PER_CU forces a
