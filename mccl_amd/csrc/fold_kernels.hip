@@ -706,8 +706,8 @@ __global__ void __launch_bounds__(kHoldBlock) fold_few_hold_kernel(FewArgs a, ui
             }
         }
     }
-    // a packet's result takes the place of its first operand (kHoldPlan: four elements per packet)
-    static_assert(C::E == 4, "the hold form keeps results where packets of four elements were");
+    // a packet's result takes the place of its first operand: four fp32 values, or eight
+    // 16-bit ones in the form they are stored in
     uint32_t lane2 = lane;
     asm volatile("" : "+v"(lane2));
 #pragma unroll
@@ -719,7 +719,12 @@ __global__ void __launch_bounds__(kHoldBlock) fold_few_hold_kernel(FewArgs a, ui
             float acc[C::E];
             combine<C>(col, acc);
             finish_pack<C>(acc, scale, has_scale != 0);
-            raw[0][u] = u32x4{__float_as_uint(acc[0]), __float_as_uint(acc[1]), __float_as_uint(acc[2]), __float_as_uint(acc[3])};
+            if constexpr (C::E == 4) {
+                raw[0][u] = u32x4{__float_as_uint(acc[0]), __float_as_uint(acc[1]), __float_as_uint(acc[2]), __float_as_uint(acc[3])};
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) raw[0][u][j] = Num<C::W>::enc(acc[2 * j]) | (Num<C::W>::enc(acc[2 * j + 1]) << 16);
+            }
         }
 #if MCCLX_TUNE_TIMELINE
     const uint64_t t_args = wall_clock64();  // here: this block has its data
@@ -732,9 +737,21 @@ __global__ void __launch_bounds__(kHoldBlock) fold_few_hold_kernel(FewArgs a, ui
     for (int u = 0; u < T; ++u) {
         const uint32_t p = (uint32_t)u * L + lane3;
         if (p < P) {
-            const float y[C::E] = {__uint_as_float(raw[0][u].x), __uint_as_float(raw[0][u].y), __uint_as_float(raw[0][u].z),
-                                   __uint_as_float(raw[0][u].w)};
-            store_pack<C, FAN>(t, has_out, has_wire, p, y, fan);
+            if constexpr (C::E == 4) {
+                const float y[C::E] = {__uint_as_float(raw[0][u].x), __uint_as_float(raw[0][u].y), __uint_as_float(raw[0][u].z),
+                                       __uint_as_float(raw[0][u].w)};
+                store_pack<C, FAN>(t, has_out, has_wire, p, y, fan);
+            } else {  // all streams 16-bit: the packed result goes out as it is
+                const u32x4 bits = raw[0][u];
+                if (has_out) MCCLX_STG(gptr<u32x4_a2>(static_cast<uint16_t*>(t.out) + p * C::E), bits);
+                if (has_wire) MCCLX_STG(gptr<u32x4_a2>(static_cast<uint16_t*>(t.wire_out) + p * C::E), bits);
+                if constexpr (FAN) {
+#pragma unroll
+                    for (int f = 0; f < MCCLX_MAX_INPUTS - C::K; ++f)
+                        if (f < fan)
+                            MCCLX_STG(gptr<u32x4_a2>(static_cast<uint16_t*>(const_cast<void*>(t.in[C::K + f])) + p * C::E), bits);
+                }
+            }
         }
     }
     if (blockIdx.x == 0) {  // the elements in front of and behind the packet grid
@@ -755,10 +772,9 @@ __global__ void __launch_bounds__(kHoldBlock) fold_few_hold_kernel(FewArgs a, ui
 #endif
 }
 
-// Plans with a reads-then-writes form: sums of two to four operands in packets of four
-// elements (fp32, or the wire-codec folds with an fp32 stream), rounding after every step.
+// Plans with a reads-then-writes form: sums of two to four operands, rounding after every step.
 template <class C>
-constexpr bool kHoldPlan = C::K >= 2 && C::K <= 4 && C::E == 4 && C::OP == MCCLX_SUM && C::ACC == MCCLX_ACC_STEP &&
+constexpr bool kHoldPlan = C::K >= 2 && C::K <= 4 && C::OP == MCCLX_SUM && C::ACC == MCCLX_ACC_STEP &&
                            C::TOPO == MCCLX_TOPO_FOLD;
 
 // Blocks of one generation: what the device holds at once of this kernel.

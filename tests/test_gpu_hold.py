@@ -9,12 +9,13 @@ import pytest
 import torch
 
 from oracle import oracle as orc
-from oracle.oracle import F32, BF16
+from oracle.oracle import F32, F16, BF16
 
 pytestmark = pytest.mark.gpu
 
-ES = {F32: 4, BF16: 2}
-KINDS = ["f32", "out_f32", "own_first", "own_last", "all_f32"]
+ES = {F32: 4, F16: 2, BF16: 2}
+KINDS = ["f32", "out_f32", "own_first", "own_last", "all_f32", "bf16", "f16"]
+PURE16 = {"bf16": BF16, "f16": F16}
 
 
 @pytest.fixture(scope="module")
@@ -53,10 +54,12 @@ def queues(env):
 
 def io_of(L, kind):
     return {"f32": L.IO_PURE, "out_f32": L.IO_OUT_F32, "own_first": L.IO_OWN_FIRST_F32,
-            "own_last": L.IO_OWN_LAST_F32, "all_f32": L.IO_ALL_F32}[kind]
+            "own_last": L.IO_OWN_LAST_F32, "all_f32": L.IO_ALL_F32, "bf16": L.IO_PURE, "f16": L.IO_PURE}[kind]
 
 
 def in_dtype(kind, j, k):
+    if kind in PURE16:
+        return PURE16[kind]
     if kind in ("f32", "all_f32") or (kind == "own_first" and j == 0) or (kind == "own_last" and j == k - 1):
         return F32
     return BF16
@@ -65,43 +68,47 @@ def in_dtype(kind, j, k):
 def build_case(env, rng, kind, k, fan, counts, in_place=False):
     """Segments with misaligned operands; returns (plan, segs for a queue, checks, keep-alive)."""
     K, L, U, oracle_fold = env
-    W = F32 if kind == "f32" else BF16
+    W = F32 if kind == "f32" else PURE16.get(kind, BF16)
+    odt = PURE16.get(kind, F32)          # the form of the outputs
     segs, checks, keep = [], [], []
     for n in counts:
         ins, ptrs, dev = [], [], []
         for j in range(k):
             dt = in_dtype(kind, j, k)
             off = int(rng.integers(0, 5))
-            a = U.rand_values(rng, n + off + 4, dt, scale=1e-2, specials=True)
+            a = U.rand_values(rng, n + off + 4, dt, scale=1e-2, specials=(dt != F16))
             t = U.to_dev(a, dt)
             ins.append((np.ascontiguousarray(a[off:off + n]), dt))
             dev.append(t)
             ptrs.append(t.data_ptr() + off * ES[dt])
         ops = [orc.encode_bf16(a) if (dt == F32 and W == BF16) else a.copy() for a, dt in ins]
         res = oracle_fold(ops, W, False, 1.0 / 3, orc.SCALE_VIEW)
-        want = orc.decode_bf16(res) if W == BF16 else res
+        want = orc.decode_bf16(res) if (W == BF16 and odt == F32) else res
         outs = []
         for f in range(fan + 1):
             off = int(rng.integers(0, 5))
-            t = torch.full((n + off + 4,), 3.0, dtype=torch.float32, device="cuda")
+            t = torch.full((n + off + 4,), 3.0, dtype=U.TORCH_DT[odt], device="cuda")
             outs.append((t, off))
-        if in_place:  # the result over an fp32 operand
-            j = next(j for j, (_, dt) in enumerate(ins) if dt == F32)
-            outs[0] = (dev[j], (ptrs[j] - dev[j].data_ptr()) // 4)
-        dest = [t.data_ptr() + off * 4 for t, off in outs]
+        if in_place:  # the result over an operand of the output's form
+            j = next(j for j, (_, dt) in enumerate(ins) if dt == odt)
+            outs[0] = (dev[j], (ptrs[j] - dev[j].data_ptr()) // ES[odt])
+        dest = [t.data_ptr() + off * ES[odt] for t, off in outs]
         segs.append(K.make_seg(dest[0], 0, ptrs + dest[1:], n))
-        checks.append((outs, n, want))
+        checks.append((outs, n, want, odt))
         keep.append(dev)
     plan = K.make_plan(W, k, io=io_of(L, kind), scale_mode=L.SCALE_VIEW, scale=1.0 / 3, fanout=fan)
     return plan, segs, checks, keep
 
 
 def check_outputs(U, checks, what, guards=True):
-    for outs, n, want in checks:
+    for outs, n, want, odt in checks:
         for f, (t, off) in enumerate(outs):
-            U.assert_same_bits(t[off:off + n], want, F32, f"{what} destination {f}")
-            if guards and t.numel() == n + off + 4 and float(t[:1].cpu()) == 3.0:
-                assert torch.all(t[:off] == 3.0) and torch.all(t[off + n:] == 3.0), what + ": wrote outside its range"
+            if odt == F16:
+                assert np.array_equal(U.bits(t[off:off + n]), want), f"{what} destination {f}"
+            else:
+                U.assert_same_bits(t[off:off + n], want, odt, f"{what} destination {f}")
+            if guards and t.numel() == n + off + 4 and float(t[:1].float().cpu()) == 3.0:
+                assert torch.all(t[:off].float() == 3.0) and torch.all(t[off + n:].float() == 3.0), what + ": wrote outside its range"
 
 
 @pytest.mark.parametrize("kind", KINDS)
@@ -115,6 +122,8 @@ def test_hold_form_gives_the_oracles_bits(env, queues, kind, k):
         pytest.skip("no such plan")
     rng = np.random.default_rng(1000 + 10 * KINDS.index(kind) + k)
     fans = [0] if kind == "out_f32" else [0, min(2, 8 - k)]
+    if kind == "f16":
+        fans = [0, 1]
     for fan in fans:
         for counts in ([1], [7], [4099], [300_007], [33, 70_001, 5], [70_001, 0, 9], [120_000, 120_001, 119_999]):
             for in_place in ((False, True) if kind != "out_f32" and fan == 0 else (False,)):
@@ -128,7 +137,8 @@ def test_hold_form_gives_the_oracles_bits(env, queues, kind, k):
     assert plain.hold_launch_count() == 0
 
 
-@pytest.mark.parametrize("kind,k,count", [("own_first", 3, 8_000_000),    # four packets per lane
+@pytest.mark.parametrize("kind,k,count", [("bf16", 3, 13_107_200),        # a 25 MiB bucket of bf16 gradients
+                                          ("own_first", 3, 8_000_000),    # four packets per lane
                                           ("own_first", 3, 9_500_000),    # five
                                           ("all_f32", 3, 6_553_600),      # the one-launch allreduce of a 25 MiB bucket
                                           ("own_last", 4, 10_000_000),
@@ -139,24 +149,26 @@ def test_hold_form_block_shapes_against_the_plain_form(env, queues, kind, k, cou
     K, L, U, _ = env
     held, plain = queues
     g = torch.Generator(device="cuda").manual_seed(count % 1000 + k)
-    W = F32 if kind == "f32" else BF16
+    W = F32 if kind == "f32" else PURE16.get(kind, BF16)
+    odt = PURE16.get(kind, F32)
     ins = []
     for j in range(k):
         t = torch.randn(count + 3, device="cuda", generator=g) * 1e-2
-        ins.append(t if in_dtype(kind, j, k) == F32 else t.to(torch.bfloat16))
+        ins.append(t if in_dtype(kind, j, k) == F32 else t.to(U.TORCH_DT[in_dtype(kind, j, k)]))
     ptrs = [t.data_ptr() + ES[in_dtype(kind, j, k)] for j, t in enumerate(ins)]   # one element past the start
     plan = K.make_plan(W, k, io=io_of(L, kind), scale_mode=L.SCALE_VIEW, scale=1.0 / 3)
     got = []
     for q in (held, plain):
-        out = torch.full((count + 2,), 7.0, device="cuda")
+        out = torch.full((count + 2,), 7.0, dtype=U.TORCH_DT[odt], device="cuda")
         before = q.hold_launch_count()
         torch.cuda.synchronize()
-        q.fold(plan, [K.make_seg(out.data_ptr() + 4, 0, ptrs, count)])
+        q.fold(plan, [K.make_seg(out.data_ptr() + ES[odt], 0, ptrs, count)])
         q.drain()
         assert q.hold_launch_count() == before + (1 if q is held else 0)
-        assert float(out[0].cpu()) == 7.0 and float(out[-1].cpu()) == 7.0
+        assert float(out[0].float().cpu()) == 7.0 and float(out[-1].float().cpu()) == 7.0
         got.append(out)
-    assert torch.equal(got[0].view(torch.int32), got[1].view(torch.int32))
+    view = torch.int32 if odt == F32 else torch.int16
+    assert torch.equal(got[0].view(view), got[1].view(view))
 
 
 def test_a_launch_wider_than_one_generation_takes_the_plain_form(env, queues):
