@@ -659,8 +659,8 @@ extern "C" MCCLX_API void mcclx_tune_timeline(void* device_buf, uint64_t slots, 
 // packets at once, folds them as they arrive, keeps the T results in registers
 // and stores them only when the launch's reads are through.  "Through" is a
 // matter of time, not of a barrier: the host knows how many bytes the launch
-// reads and passes the moment (in ticks of the 100 MHz wall clock, counted from
-// the block's own start) before which no lane stores.  A gate that is too late
+// reads and passes the moment (in ticks of the device's wall clock, 100 MHz on
+// gfx950, counted from the block's own start) before which no lane stores.  A gate that is too late
 // costs its excess, one that is too early lets writes into the reads again --
 // results do not depend on it.  C2 (78.6 MB per launch): 14.1 -> 12.9 us.
 //
