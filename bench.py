@@ -12,11 +12,20 @@ from): per bucket element 4 B own fp32 read + 2 x 2 B bf16 peer reads + 4 B fp32
 write = 12 B  ->  78,643,200 B.
 
 The K timed steps are recorded into one HIP graph and replayed with a single
-submission, so the host's launch cost is not part of the measurement (the
-warm-up replays the same graph, i.e. max(W, K) untimed steps); steps
-rotate over several distinct copies of the workload (> 512 MiB in total) so the
-256 MiB Infinity Cache cannot serve the reads ("cold", the headline); the same
-loop over one copy is reported as "warm".
+submission (the warm-up replays the same graph, i.e. max(W, K) untimed steps).
+Two brackets around exactly K steps each:
+  * `value` / `ms_per_step`: the wall clock around one replay, queue drained and
+    device synchronised on both sides -- it includes what the host pays to submit
+    a graph, which does not shrink with K;
+  * `roofline`: HIP events on the reduce queue around one replay that is enqueued
+    directly behind the warm-up replay, so that the start event is stamped when
+    the warm-up ends and the timed launches are already queued behind it.  (With
+    a drained queue in front, the start event is stamped at once and the device
+    then idles while the host submits the replay: some 10 us that are the host's,
+    not the kernel's, and that weigh 0.5 us per step at K = 20 and 0.05 at K = 200.)
+Steps rotate over several distinct copies of the workload (> 512 MiB in total) so
+the 256 MiB Infinity Cache cannot serve the reads ("cold", the headline); the
+same loop over one copy is reported as "warm".
 
 Prints ONE JSON line.
 """
@@ -49,7 +58,7 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--timeline", action="store_true",
                     help="instead of the JSON line, print where the time of one C2 launch goes: every block's "
-                         "start and end stamps from the instrumented build (python -m mccl_amd.build --timeline)")
+                         "start and end stamps from the measurement build (python -m mccl_amd.build --bench)")
     return ap.parse_args()
 
 
@@ -62,14 +71,14 @@ def main():
 
     import numpy as np
     import torch
-    from mccl_amd.build import ensure_built, TIMELINE_LIB_PATH
+    from mccl_amd.build import ensure_built, BENCH_LIB_PATH
     ensure_built()
     if args.timeline:
-        if not os.path.exists(TIMELINE_LIB_PATH):
-            print("bench.py --timeline needs the instrumented build: python -m mccl_amd.build --timeline",
+        if not os.path.exists(BENCH_LIB_PATH):
+            print("bench.py --timeline needs the measurement build: python -m mccl_amd.build --bench",
                   file=sys.stderr)
             sys.exit(2)
-        os.environ["MCCLX_LIBRARY"] = TIMELINE_LIB_PATH
+        os.environ["MCCLX_LIBRARY"] = BENCH_LIB_PATH
     from mccl_amd import _lib as L
     from mccl_amd import kernels as K
     from mccl_amd import harness as H
@@ -138,34 +147,39 @@ def main():
     del outs
 
     # ---- timed loops, each recorded into one graph
-    def record(n_steps, seg_fn):
-        q.graph_begin()
+    def record(n_steps, seg_fn, qu):
+        qu.graph_begin()
         for i in range(n_steps):
             seg_fn(i)
-        return q.graph_end()
+        return qu.graph_end()
 
-    def timed(graph):
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        q.timer_begin()
-        q.graph_launch(graph)
-        ms_dev = q.timer_end()
-        torch.cuda.synchronize()
-        return ms_dev, (time.perf_counter() - t0) * 1e3
-
-    def measure(seg_fn, steps, warmup):
-        """Untimed warm-up, then exactly `steps` timed steps.  The warm-up replays the
-        same recorded graph (so at least `warmup` steps, in whole replays): the first
-        replays of a freshly instantiated graph run about 4 % slower per kernel than
-        later ones, which is a property of the launch path, not of the kernel.  The
-        data stays cold either way: every replay walks all rotating copies again."""
+    def measure(seg_fn, steps, warmup, wall=False, queue=None):
+        """Untimed warm-up, then exactly `steps` timed steps; returns (device ms, wall ms or None).
+        The warm-up replays the same recorded graph (so at least `warmup` steps, in whole
+        replays, and at least one replay): the first replays of a freshly instantiated graph
+        run about 4 % slower per kernel than later ones, which is a property of the launch
+        path, not of the kernel.  The data stays cold either way: every replay walks all
+        rotating copies again.  Device time: events on the reduce queue around a replay
+        enqueued directly behind the warm-up.  Wall time (`wall=True`): a second replay of
+        the same K steps, bracketed by a drain and a device synchronisation on both sides."""
+        qu = queue or q
         torch.cuda.synchronize()  # inputs made by torch ops are complete before the queue reads them
-        gk = record(steps, seg_fn)
-        for _ in range(max(1, -(-warmup // steps)) if warmup > 0 else 0):
-            q.graph_launch(gk)
-        q.drain()
-        ms_dev, ms_wall = timed(gk)
-        q.graph_destroy(gk)
+        gk = record(steps, seg_fn, qu)
+        for _ in range(max(1, -(-warmup // steps))):
+            qu.graph_launch(gk)
+        qu.timer_begin()
+        qu.graph_launch(gk)
+        ms_dev = qu.timer_end()
+        ms_wall = None
+        if wall:
+            qu.drain()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            qu.graph_launch(gk)
+            qu.drain()
+            torch.cuda.synchronize()
+            ms_wall = (time.perf_counter() - t0) * 1e3
+        qu.graph_destroy(gk)
         return ms_dev, ms_wall
 
     cold = lambda i: q.fold(plan, step_segs(i % args.sets, out_tensors=results[i % args.sets]))
@@ -173,7 +187,7 @@ def main():
     if args.timeline:
         timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure, bytes_per_step)
         return
-    cold_dev, cold_wall = measure(cold, args.steps, args.warmup)
+    cold_dev, cold_wall = measure(cold, args.steps, args.warmup, wall=True)
     warm_dev, _ = measure(warm, args.steps, args.warmup)
 
     gbs = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
@@ -202,7 +216,10 @@ def main():
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": C2_MEASURED_TRAFFIC_BYTES,
                      "kernel": "fold_few_hold_kernel<bf16, own-first fp32, k=3; 4 packets per lane, 512-lane blocks>", "kernel_us": round(kernel_us, 2)},
     }
-    extra = {"warm_GBps": round(gbs(bytes_per_step, warm_dev / args.steps), 1),
+    lat_ticks, bpt, measured = q.hold_model()
+    extra = {"hold_gate": {"latency_ticks": lat_ticks, "bytes_per_tick": bpt, "measured_on_this_device": measured,
+                           "ticks_for_this_launch": lat_ticks + (numel * 8) // bpt},
+             "warm_GBps": round(gbs(bytes_per_step, warm_dev / args.steps), 1),
              "warm_kernel_us": round(warm_dev / args.steps * 1e3, 2),
              "pct_of_hbm_peak_cold": round(100 * achieved / HBM_PEAK_GBS, 2)}
 
@@ -288,7 +305,7 @@ def timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure,
     pr = out.append
     pr("C2 fused fold -- timeline of one launch from per-block time stamps, MI355X (gfx950)")
     pr("")
-    pr("Command: python -m mccl_amd.build --timeline   (here, once)   then on the GPU box:   python bench.py --timeline")
+    pr("Command: python -m mccl_amd.build --bench   (here, once)   then on the GPU box:   python bench.py --timeline")
     pr("Every block of the fold <bf16, own-first fp32, k=3> records wall_clock64() (100 MHz, 10 ns ticks) at its first")
     pr("instruction, at a second point, and after its last store was issued.  16 consecutive launches (cold = rotating 8")
     pr("copies of the workload, 944 MB + 629 MB of results) are recorded into one HIP graph; figures are means over")
@@ -554,12 +571,37 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
     # one-directional ceilings at the bucket launch's own footprint (78,643,200 B, cold-rotated): a
     # launch that only reads that many bytes and one that only writes them
     fp = numel * 12
-    probe = torch.randint(0, 256, (8 * fp,), dtype=torch.uint8, device="cuda")
-    for write, name in ((False, "read_only"), (True, "write_only")):
-        ms, _ = measure(lambda i, write=write: q.probe_stream(probe.data_ptr() + (i % 8) * fp, fp, write), steps, warm)
-        out[f"{name}_same_footprint_us"] = round(ms / steps * 1e3, 2)
-        out[f"{name}_same_footprint_GBps"] = round(gbs(fp, ms / steps), 1)
-    del probe
+    if L.bench_lib() is not None:  # the probe launch is the measurement build's (python -m mccl_amd.build --bench)
+        probe = torch.randint(0, 256, (8 * fp,), dtype=torch.uint8, device="cuda")
+        for write, name in ((False, "read_only"), (True, "write_only")):
+            ms, _ = measure(lambda i, write=write: q.probe_stream(probe.data_ptr() + (i % 8) * fp, fp, write), steps, warm)
+            out[f"{name}_same_footprint_us"] = round(ms / steps * 1e3, 2)
+            out[f"{name}_same_footprint_GBps"] = round(gbs(fp, ms / steps), 1)
+        del probe
+    else:
+        out["read_only_same_footprint_us"] = out["write_only_same_footprint_us"] = None
+
+    # the gate of the hold form: the rate measured on this device when the library started, against
+    # gates a few per cent earlier and later (each on a context of its own, made with the override)
+    lat_ticks, bpt, measured = q.hold_model()
+    sweep = {}
+    saved = os.environ.get("MCCLX_HOLD_BYTES_PER_TICK")
+    try:
+        for pct in (-6, -3, 0, 3, 6):
+            os.environ["MCCLX_HOLD_BYTES_PER_TICK"] = str(int(bpt * (1 - pct / 100.0)))
+            qq = K.ReduceQueue(0)
+            try:
+                ms, _ = measure(lambda i: qq.fold(plan, step_segs(i % sets, out_tensors=results[i % sets])), steps, warm,
+                                queue=qq)
+            finally:
+                qq.close()
+            sweep[f"{pct:+d}%"] = round(ms / steps * 1e3, 2)
+    finally:
+        if saved is None:
+            os.environ.pop("MCCLX_HOLD_BYTES_PER_TICK", None)
+        else:
+            os.environ["MCCLX_HOLD_BYTES_PER_TICK"] = saved
+    out["c2_fold_us_by_gate_shift"] = sweep  # "+3%": the gate 3 % later than the one the library uses
 
     # the headline launch in the plain form (one block per tile, loads then stores, reads and writes
     # mixed on the memory bus) instead of the hold form (all loads, then all stores) it takes by default

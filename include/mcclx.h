@@ -32,10 +32,13 @@ extern "C" {
 
 #define MCCLX_API __attribute__((visibility("default")))
 /* 2: mcclx_plan.flags (was a reserved field that had to be 0), mcclx_fold_batched_noalloc,
- *    mcclx_probe_stream.  Layouts of version 1 callers stay valid.
+ *    mcclx_probe_stream (gone again in 4).  Layouts of version 1 callers stay valid.
  * 3: MCCLX_IO_ALL_F32, MCCLX_REPLAY_DIRECT, mcclx_set_hold, mcclx_hold_launch_count.
+ *    Layouts unchanged.
+ * 4: mcclx_hold_model; the measurement aids mcclx_probe_stream and mcclx_timer_begin / _end
+ *    left the library (the measurement build declares its own in mcclx_bench.h).
  *    Layouts unchanged. */
-#define MCCLX_ABI_VERSION 3
+#define MCCLX_ABI_VERSION 4
 #define MCCLX_MAX_INPUTS 8 /* inputs one launch folds; wider worlds chain launches */
 
 /* ---- codes ---------------------------------------------------------------- */
@@ -128,6 +131,13 @@ MCCLX_API uint64_t mcclx_launch_count(mcclx_ctx* ctx);
 MCCLX_API int mcclx_set_hold(mcclx_ctx* ctx, int enabled);
 /* Diagnostic: launches of this context that took the hold form. */
 MCCLX_API uint64_t mcclx_hold_launch_count(mcclx_ctx* ctx);
+/* Diagnostic: the model behind that time -- no store before `latency_ticks` +
+ * bytes read / `bytes_per_tick` ticks of a 100 MHz clock after a block's start.
+ * The rate is measured on the device when the first context of a process is made
+ * on it (two read-only launches over scratch memory; MCCLX_HOLD_CALIBRATE=0 keeps
+ * the built-in value).  Returns 1 if this context's rate was measured, 0 if it is
+ * the built-in value or an MCCLX_HOLD_BYTES_PER_TICK override. */
+MCCLX_API int mcclx_hold_model(mcclx_ctx* ctx, uint32_t* latency_ticks, uint32_t* bytes_per_tick);
 
 /* ---- the reference's four kernel entry points, one to one ------------------- */
 
@@ -227,9 +237,12 @@ MCCLX_API int mcclx_fold_batched(mcclx_ctx* ctx, const mcclx_plan* plan, const m
  * fill from their own arguments -- the whole call is kernel launches only.
  * More than MCCLX_NOALLOC_MAX_SEGS segments are refused with MCCLX_ERR_INVALID.
  * Every call on a GPU shares that GPU's array: calls on one context are
- * ordered by its queue, calls that overlap on one GPU from different contexts
- * race.  Nothing in the array needs to start at zero; each call overwrites the
- * part it reads. */
+ * ordered by its queue; a call that enters while another thread's call on the
+ * same GPU is still filling the array is refused with MCCLX_ERR_STATE; launches
+ * of different contexts that are both queued and overlap on the device race.
+ * Nothing in the array needs to start at zero; each call overwrites the part it
+ * reads.  Launches of up to 32 segments of similar length carry their
+ * descriptors in the kernel arguments and do not touch the array. */
 #define MCCLX_NOALLOC_MAX_SEGS 1024
 MCCLX_API int mcclx_fold_batched_noalloc(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs,
                                uint32_t nseg);
@@ -269,15 +282,6 @@ MCCLX_API int mcclx_stream_wait_queue(mcclx_ctx* ctx, void* consumer_stream);
 MCCLX_API int mcclx_event_record(mcclx_ctx* ctx, uint64_t* ticket);
 MCCLX_API int mcclx_event_query(mcclx_ctx* ctx, uint64_t ticket, int* done);
 MCCLX_API int mcclx_event_wait(mcclx_ctx* ctx, uint64_t ticket);
-/* Device-time bracket on the queue (hipEvents), for measurement. */
-MCCLX_API int mcclx_timer_begin(mcclx_ctx* ctx);
-MCCLX_API int mcclx_timer_end(mcclx_ctx* ctx, float* elapsed_ms);
-
-/* Measurement aid: one launch that only reads (write = 0) or only writes
- * (write = 1) nbytes of `buf` (4-byte aligned; its contents are unspecified
- * afterwards) with the copy kernel's access shape -- the one-directional
- * ceilings a fold launch of the same footprint is compared with. */
-MCCLX_API int mcclx_probe_stream(mcclx_ctx* ctx, void* buf, uint64_t nbytes, int write);
 
 /* ---- launch graphs ---------------------------------------------------------- */
 
@@ -286,7 +290,7 @@ MCCLX_API int mcclx_probe_stream(mcclx_ctx* ctx, void* buf, uint64_t nbytes, int
  * single submission -- the HIP form of the reference's "many launches, one
  * command buffer" batch (MetalKernels.mm:559-577).  Between graph_begin and
  * graph_end every launch on this context is recorded instead of executed
- * (queue_drain, event_* and timer_* are refused while recording).  Buffers
+ * (queue_drain and event_* are refused while recording).  Buffers
  * named by recorded launches must stay valid for the graph's lifetime. */
 typedef struct mcclx_graph mcclx_graph;
 MCCLX_API int mcclx_graph_begin(mcclx_ctx* ctx);

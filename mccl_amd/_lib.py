@@ -76,6 +76,7 @@ SIGNATURES = {
     "mcclx_launch_count": (_u64, [_vp]),
     "mcclx_hold_launch_count": (_u64, [_vp]),
     "mcclx_set_hold": (_i, [_vp, _i]),
+    "mcclx_hold_model": (_i, [_vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "mcclx_reduce": (_i, [_vp, _vp, _vp, _i, _u64, _i]),
     "mcclx_scale": (_i, [_vp, _vp, _i, _u64, _d, _i]),
     "mcclx_accumulate_scale": (_i, [_vp, _vp, _vp, _i, _u64, _d]),
@@ -88,15 +89,12 @@ SIGNATURES = {
     "mcclx_fold_batched_noalloc": (_i, [_vp, C.POINTER(Plan), C.POINTER(Seg), C.c_uint32]),
     "mcclx_copy": (_i, [_vp, _vp, _vp, _u64]),
     "mcclx_copy_batched": (_i, [_vp, C.POINTER(CopyDesc), C.c_uint32]),
-    "mcclx_probe_stream": (_i, [_vp, _vp, _u64, _i]),
     "mcclx_queue_drain": (_i, [_vp]),
     "mcclx_queue_wait_stream": (_i, [_vp, _vp]),
     "mcclx_stream_wait_queue": (_i, [_vp, _vp]),
     "mcclx_event_record": (_i, [_vp, C.POINTER(C.c_uint64)]),
     "mcclx_event_query": (_i, [_vp, _u64, C.POINTER(C.c_int)]),
     "mcclx_event_wait": (_i, [_vp, _u64]),
-    "mcclx_timer_begin": (_i, [_vp]),
-    "mcclx_timer_end": (_i, [_vp, C.POINTER(C.c_float)]),
     "mcclx_graph_begin": (_i, [_vp]),
     "mcclx_graph_end": (_i, [_vp, _pp]),
     "mcclx_graph_launch": (_i, [_vp, _vp]),
@@ -150,6 +148,27 @@ def lib() -> C.CDLL:
             fn.argtypes = args
         _lib = L
     return _lib
+
+
+BENCH_LIB_PATH = os.path.join(HERE, "libmcclx_bench.so")
+_bench = None
+
+
+def bench_lib():
+    """The measurement build (include/mcclx_bench.h), or None when it has not been built
+    (`python -m mccl_amd.build --bench`).  Loaded next to the shipped library; only its
+    probe launch, which takes a raw stream, is used from here."""
+    global _bench
+    if _bench is None:
+        import torch  # noqa: F401  (one HIP runtime per process, see lib())
+        if not os.path.exists(BENCH_LIB_PATH):
+            return None
+        B = C.CDLL(BENCH_LIB_PATH)
+        B.mcclx_bench_probe.restype = _i
+        B.mcclx_bench_probe.argtypes = [_vp, _vp, _u64, _i]
+        B.mcclx_last_error.restype = C.c_char_p
+        _bench = B
+    return _bench
 
 
 def last_error() -> str:

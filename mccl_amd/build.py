@@ -52,11 +52,8 @@ def needs_build() -> bool:
     return not os.path.exists(LIB_PATH) or os.path.getmtime(LIB_PATH) < _newest_source_mtime()
 
 
-def build(force: bool = True, verbose: bool = False) -> str:
-    """Compile every source and link mccl_amd/libmcclx.so.  Returns its path."""
-    if not force and not needs_build():
-        return LIB_PATH
-    os.makedirs(OBJ_DIR, exist_ok=True)
+def _compile_and_link(out_path: str, obj_dir: str, extra_flags, verbose: bool) -> str:
+    os.makedirs(obj_dir, exist_ok=True)
     cc = hipcc()
     procs = []
     objs = []
@@ -67,9 +64,9 @@ def build(force: bool = True, verbose: bool = False) -> str:
         else:
             units.append((src, os.path.splitext(src)[0] + ".o", []))
     for src, objname, extra in units:
-        obj = os.path.join(OBJ_DIR, objname)
+        obj = os.path.join(obj_dir, objname)
         objs.append(obj)
-        cmd = [cc] + HIPCC_FLAGS + extra + (["-x", "hip"] if src.endswith(".cpp") else []) + \
+        cmd = [cc] + HIPCC_FLAGS + list(extra_flags) + extra + (["-x", "hip"] if src.endswith(".cpp") else []) + \
               ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -81,13 +78,20 @@ def build(force: bool = True, verbose: bool = False) -> str:
             raise RuntimeError(f"hipcc failed on {src}:\n{out}")
         if verbose and out.strip():
             print(out, flush=True)
-    tmp = LIB_PATH + ".tmp"
+    tmp = out_path + ".tmp"
     link = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + objs
     r = subprocess.run(link, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stdout}")
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    os.replace(tmp, out_path)
+    return out_path
+
+
+def build(force: bool = True, verbose: bool = False) -> str:
+    """Compile every source and link mccl_amd/libmcclx.so.  Returns its path."""
+    if not force and not needs_build():
+        return LIB_PATH
+    return _compile_and_link(LIB_PATH, OBJ_DIR, [], verbose)
 
 
 BACKEND_DIR = os.path.join(CSRC, "backend")
@@ -147,24 +151,18 @@ def build_backend(verbose: bool = False) -> str:
     return out_path
 
 
-TIMELINE_LIB_PATH = os.path.join(HERE, "libmcclx_timeline.so")
+BENCH_LIB_PATH = os.path.join(HERE, "libmcclx_bench.so")
 
 
-def build_timeline(verbose: bool = False) -> str:
-    """The tuning build bench.py --timeline loads: the same sources with
-    -DMCCLX_TUNE_TIMELINE=1 (every block of a by-value fold launch records its start
-    and end times) and only the measured plans instantiated, in one translation unit
-    per source.  Written to mccl_amd/libmcclx_timeline.so; the shipped library is
-    not touched."""
-    cc = hipcc()
-    cmd = [cc] + HIPCC_FLAGS + ["-DMCCLX_TUNE_TIMELINE=1", "-DMCCLX_TUNE_MINIMAL=1", "-x", "hip", "-shared",
-                                "-o", TIMELINE_LIB_PATH] + [os.path.join(CSRC, s) for s in SOURCES]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed on the timeline build:\n{r.stdout}")
-    return TIMELINE_LIB_PATH
+def build_bench(verbose: bool = False) -> str:
+    """The measurement build (include/mcclx_bench.h), on request only
+    (`python -m mccl_amd.build --bench`): the same sources with
+    -DMCCLX_TUNE_TIMELINE=1 -- every block of a by-value fold launch can record its
+    start, data and end times, and the read-only / write-only probe launch is
+    exported.  bench.py takes its one-directional ceilings from it and
+    `bench.py --timeline` runs on it; without it those figures are left out.
+    Written to mccl_amd/libmcclx_bench.so; the shipped library is not touched."""
+    return _compile_and_link(BENCH_LIB_PATH, os.path.join(ROOT, "build", "mcclx_bench"), ["-DMCCLX_TUNE_TIMELINE=1"], verbose)
 
 
 def ensure_built() -> None:
@@ -177,5 +175,5 @@ if __name__ == "__main__":
     print(build(force="--force" in sys.argv or needs_build(), verbose=True))
     if "--backend" in sys.argv:
         print(build_backend(verbose=True))
-    if "--timeline" in sys.argv:
-        print(build_timeline(verbose=True))
+    if "--bench" in sys.argv:
+        print(build_bench(verbose=True))

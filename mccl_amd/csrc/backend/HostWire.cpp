@@ -1,6 +1,7 @@
 #include "backend/HostWire.hpp"
 
 #include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
 
 #include <algorithm>
 #include <cstring>
@@ -12,7 +13,10 @@ namespace mccl {
 
 struct HostWire::Ctx {
     mcclx_ctx* ctx = nullptr;
+    hipEvent_t t0 = nullptr, t1 = nullptr;  // device-time bracket around the fold, for the statistics
     ~Ctx() {
+        if (t0) (void)hipEventDestroy(t0);
+        if (t1) (void)hipEventDestroy(t1);
         if (ctx) mcclx_destroy(ctx);
     }
 };
@@ -245,10 +249,17 @@ void HostWire::allreduce(void* tensor, int dtype, uint64_t numel, int op, int al
             s.out = at(tensor, mine->start * ts);
             if (codec) s.wire_out = at(send_dev, mine->start * 2);  // the reduced chunk as it travels on
         }
-        check_rc(mcclx_timer_begin(ctx));
+        hipStream_t qs = static_cast<hipStream_t>(mcclx_queue_stream(ctx));
+        if (!ctx_->t0) {
+            MCCL_CHECK(hipEventCreate(&ctx_->t0) == hipSuccess && hipEventCreate(&ctx_->t1) == hipSuccess,
+                       "host wire: hipEventCreate failed");
+        }
+        MCCL_CHECK(hipEventRecord(ctx_->t0, qs) == hipSuccess, "host wire: hipEventRecord failed");
         check_rc(mcclx_fold_batched(ctx, &plan, &s, 1));
         float ms = 0.f;
-        check_rc(mcclx_timer_end(ctx, &ms));
+        MCCL_CHECK(hipEventRecord(ctx_->t1, qs) == hipSuccess && hipEventSynchronize(ctx_->t1) == hipSuccess &&
+                       hipEventElapsedTime(&ms, ctx_->t0, ctx_->t1) == hipSuccess,
+                   "host wire: timing the fold failed");
         stats_.fold_ms = ms;
         stats_.fold_elems = mine->count;
         stats_.fold_peer_bytes = static_cast<uint64_t>(N - 1) * mine->count * es;

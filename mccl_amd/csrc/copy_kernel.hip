@@ -9,31 +9,20 @@
 
 #include "fold_launch.h"
 
-#ifndef MCCLX_TUNE_COPY_U
-#define MCCLX_TUNE_COPY_U 1
-#endif
-#ifndef MCCLX_TUNE_COPY_NT
-#define MCCLX_TUNE_COPY_NT 1  // every byte is touched once: non-temporal loads and stores
-#endif
-
 namespace mcclx {
 namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #define MCCLX_GLOBAL __attribute__((address_space(1)))
-#if MCCLX_TUNE_COPY_NT
+// every byte is touched once: non-temporal loads and stores
 #define COPY_LD(p) __builtin_nontemporal_load(p)
 #define COPY_ST(p, v) __builtin_nontemporal_store((v), (p))
-#else
-#define COPY_LD(p) (*(p))
-#define COPY_ST(p, v) (*(p) = (v))
-#endif
 // the widest alignment both pointers share decides the packet type
 template <int A> struct Packet;
 template <> struct Packet<4> { typedef u32x4 type __attribute__((aligned(4))); };
 template <> struct Packet<2> { typedef u32x4 type __attribute__((aligned(2))); };
 template <> struct Packet<1> { typedef u32x4 type __attribute__((aligned(1))); };
 constexpr int kBlock = 256;
-constexpr int kU = MCCLX_TUNE_COPY_U;
+constexpr int kU = 1;  // packets per lane
 
 // Up to kFewCopies copies with their descriptors in the kernel arguments:
 // blockIdx.y picks the copy, blockIdx.x one tile of kU * kBlock packets of 16

@@ -38,56 +38,20 @@
 namespace mcclx {
 namespace {
 
-// Build-time tuning knobs (defaults are the measured best on MI355X).
-#ifndef MCCLX_TUNE_BLOCK
-#define MCCLX_TUNE_BLOCK 512
-#endif
-#ifndef MCCLX_TUNE_U
-#define MCCLX_TUNE_U 0  // 0: the measured best per plan (Cfg::U)
-#endif
-#ifndef MCCLX_TUNE_NT_LOAD
-#define MCCLX_TUNE_NT_LOAD 1
-#endif
-#ifndef MCCLX_TUNE_NT_STORE
-#define MCCLX_TUNE_NT_STORE 1
-#endif
-#ifndef MCCLX_TUNE_HWCVT
-#define MCCLX_TUNE_HWCVT 1  // 1: v_cvt_pk_bf16_f32 + NaN fix-up; 0: integer rounding
-#endif
-#ifndef MCCLX_TUNE_XCD
-#define MCCLX_TUNE_XCD 0    // N > 0: give each of N XCDs one contiguous N-th of a segment's tiles
-#endif
-#ifndef MCCLX_TUNE_PEEL
-#define MCCLX_TUNE_PEEL 1   // scalar head peel up to the output's 128-byte boundary
-#endif
-
-constexpr int kBlock = MCCLX_TUNE_BLOCK;  // threads per block of folds that mix fp32 and 16-bit streams
-#ifndef MCCLX_TUNE_WIDE_BLOCK
-#define MCCLX_TUNE_WIDE_BLOCK 64
-#endif
-#ifndef MCCLX_TUNE_WIDE_U
-#define MCCLX_TUNE_WIDE_U 1
-#endif
-#ifndef MCCLX_TUNE_WIDE_MINK
-#define MCCLX_TUNE_WIDE_MINK 2
-#endif
-#ifndef MCCLX_TUNE_F32_BLOCK
-#define MCCLX_TUNE_F32_BLOCK 64
-#endif
-#ifndef MCCLX_TUNE_ALLF32_BLOCK
-#define MCCLX_TUNE_ALLF32_BLOCK 64  // every operand fp32, encoded in registers (MCCLX_IO_ALL_F32)
-#endif
-// Block size by plan, each measured on MI355X.  Folds whose streams all have one
-// element size -- all 16-bit (16 bytes per lane and operand) or all fp32 -- run
-// one-wavefront blocks with one packet per lane: a 512-lane block keeps its wave
-// slots until the last of its loads is back, 64-lane blocks turn them over eight
-// times as often (two to eight 16-bit operands of 512 MiB: +5...9 %, fp32
-// operands: +3...4 %; launches of a few MB are level; fp32 operands encoded in
-// registers, MCCLX_IO_ALL_F32: +7 % on 256 MiB tensors, +1.5 % on 25 MiB ones).
-// Folds that mix an fp32 stream with 16-bit peers (the wire-codec folds) are
-// fastest at 512, and so are one-operand passes.
-constexpr int kWideBlock = MCCLX_TUNE_WIDE_BLOCK;
-constexpr int kWideU = MCCLX_TUNE_WIDE_U;
+// Launch shapes, each measured on MI355X.
+constexpr int kBlock = 512;  // threads per block of folds that mix fp32 and 16-bit streams, and of one-operand passes
+// Folds whose streams all have one element size -- all 16-bit (16 bytes per lane
+// and operand) or all fp32 -- run one-wavefront blocks with one packet per lane:
+// a 512-lane block keeps its wave slots until the last of its loads is back,
+// 64-lane blocks turn them over eight times as often (two to eight 16-bit
+// operands of 512 MiB: +5...9 %, fp32 operands: +3...4 %; launches of a few MB
+// are level; fp32 operands encoded in registers, MCCLX_IO_ALL_F32: +7 % on
+// 256 MiB tensors, +1.5 % on 25 MiB ones).
+constexpr int kWideBlock = 64;
+constexpr int kWideU = 1;
+constexpr int kWideMinK = 2;   // all-16-bit folds of this many operands or more take the one-wavefront shape
+constexpr int kF32Block = 64;
+constexpr int kAllF32Block = 64;
 
 // Every operand lives in global memory (HBM or host memory mapped into the
 // device).  Pointers that reach a kernel through a descriptor table are
@@ -108,30 +72,17 @@ typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 typedef u32x2 u32x2_a2 __attribute__((aligned(2)));
 // Loads and stores of one packet through the under-aligned pointer types
 // (macros, so the typedef's alignment stays attached to the access).
-#if MCCLX_TUNE_NT_LOAD
+// (the hold form with ordinary stores: 14.85 us for a launch the non-temporal ones run in 13.1 us)
 #define MCCLX_LDG(p) __builtin_nontemporal_load(p)
-#else
-#define MCCLX_LDG(p) (*(p))
-#endif
-#if MCCLX_TUNE_NT_STORE
 #define MCCLX_STG(p, v) __builtin_nontemporal_store((v), (p))
-#else
-#define MCCLX_STG(p, v) (*(p) = (v))
-#endif
 
 // ---------------------------------------------------------------- rounding
 
 // fp32 -> bf16 round-to-nearest-even, NaN -> 0x7FC0, result kept as the fp32
 // whose low half is zero (torch/headeronly/util/BFloat16.h:100-114).
 __device__ __forceinline__ uint32_t bf16_round_bits(float x) {
-#if MCCLX_TUNE_HWCVT
-    uint32_t r = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)x) << 16;
+    uint32_t r = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)x) << 16;  // v_cvt_pk_bf16_f32
     return (x != x) ? 0x7FC00000u : r;
-#else
-    uint32_t u = __float_as_uint(x);
-    uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
-    return ((u & 0x7FFFFFFFu) > 0x7F800000u) ? 0x7FC00000u : r;
-#endif
 }
 
 template <int W> struct Num;  // arithmetic dtype traits
@@ -162,17 +113,12 @@ template <> struct Num<MCCLX_BF16> {
     // two values per v_cvt_pk_bf16_f32; a NaN whose quiet bit is set (every NaN an
     // add, a multiply or a decoded bf16 operand can hand over) converts to a NaN
     template <int E> __device__ static __forceinline__ void round_mid(float (&x)[E]) {
-#if MCCLX_TUNE_HWCVT
 #pragma unroll
         for (int j = 0; j < E; j += 2) {
             const uint32_t u = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{x[j], x[j + 1]}, bf16x2));
             x[j] = __uint_as_float(u << 16);
             x[j + 1] = __uint_as_float(u & 0xFFFF0000u);
         }
-#else
-#pragma unroll
-        for (int j = 0; j < E; ++j) x[j] = rnd(x[j]);
-#endif
     }
     template <int E> __device__ static __forceinline__ void canon(float (&x)[E]) {
 #pragma unroll
@@ -233,15 +179,14 @@ struct Cfg {
     // no grid-stride looping): one packet per lane streams fastest for folds with
     // an fp32 stream; all-16-bit plans and the one-input codec passes (encode,
     // decode), whose lanes move few bytes, gain 4-12 % from two.
-    static constexpr bool kWide = (E == 8 && K >= MCCLX_TUNE_WIDE_MINK);
-    static constexpr int U = MCCLX_TUNE_U ? MCCLX_TUNE_U
-                             : kWide ? kWideU
+    static constexpr bool kWide = (E == 8 && K >= kWideMinK);
+    static constexpr int U = kWide ? kWideU
                              : (TOPO == MCCLX_TOPO_BINOMIAL) ? 1
                              : ((E == 8 || (K == 1 && IO != MCCLX_IO_PURE)) ? 2 : 1);
     static constexpr bool kDecode = (K == 1 && IO == MCCLX_IO_OUT_F32);  // bf16 -> fp32 cast: +3 % at 64
     static constexpr int BLOCK = kWide ? kWideBlock
-                                 : ((W == MCCLX_F32 && K >= 2) || kDecode) ? MCCLX_TUNE_F32_BLOCK
-                                 : (IO == MCCLX_IO_ALL_F32 && K >= 2) ? MCCLX_TUNE_ALLF32_BLOCK : kBlock;  // threads per block
+                                 : ((W == MCCLX_F32 && K >= 2) || kDecode) ? kF32Block
+                                 : (IO == MCCLX_IO_ALL_F32 && K >= 2) ? kAllF32Block : kBlock;  // threads per block
 };
 
 typedef u32x4 RawPack;  // one packet of one operand: 16 B, or 8 B in .xy (16-bit operand, E = 4)
@@ -482,16 +427,11 @@ __device__ __forceinline__ void fold_packs(const SegArgs& s, bool has_out, bool 
 // buffer the widest stores go to.
 template <class C>
 __device__ __forceinline__ uint32_t head_elems(const SegArgs& s) {
-#if MCCLX_TUNE_PEEL
     const bool wide_out = (C::W == MCCLX_F32 || C::kOutF32) && s.out;
     const uint32_t a = (uint32_t)reinterpret_cast<uintptr_t>(s.out ? s.out : s.wire_out);
     const uint32_t mis = a & 127u;
     const uint32_t h = mis ? (128u - mis) >> (wide_out ? 2 : 1) : 0u;
     return s.count < h ? (uint32_t)s.count : h;
-#else
-    (void)s;
-    return 0;
-#endif
 }
 
 // Every pointer of the segment moved `elems` elements on (null outputs become
@@ -595,16 +535,11 @@ __device__ __forceinline__ void fold_few_body(const FewArgs& a) {
     const uint64_t t_args = wall_clock64();
 #endif
     const uint64_t span = (uint64_t)C::U * C::BLOCK;
-#if MCCLX_TUNE_XCD
-    // workgroups go to the XCDs round robin: block b runs on XCD b % N
-    const uint32_t per = grid / MCCLX_TUNE_XCD;  // the grid is a multiple of N
-    const uint32_t tile = (blockIdx.x % MCCLX_TUNE_XCD) * per + blockIdx.x / MCCLX_TUNE_XCD;
-    fold_tile<C, FAN>(s, scale, has_scale != 0, (uint64_t)tile * span, tile == 0, fan);
-#else
-    // one tile per block, no loop: the launch sizes the grid to the longest segment
+    // one tile per block, no loop: the launch sizes the grid to the longest segment.  Blocks are
+    // dispatched in address order (giving each XCD one contiguous part of a segment instead was
+    // level on a 25 MiB bucket and 3.5-9 % slower on large operands).
     (void)grid;
     fold_tile<C, FAN>(s, scale, has_scale != 0, (uint64_t)blockIdx.x * span, blockIdx.x == 0, fan);
-#endif
 #if MCCLX_TUNE_TIMELINE
     if (a.timeline && threadIdx.x == 0) {
         TimelineRecord r;
@@ -634,20 +569,10 @@ template <class C>
 __global__ void __launch_bounds__(C::BLOCK) fold_few_fan_kernel(FewArgs a) { fold_few_body<C, true>(a); }
 
 #if MCCLX_TUNE_TIMELINE
-// Where the next by-value launches put their records: a caller-provided device
-// buffer cut into `slots` regions of `per_slot` records, used round robin.
-static TimelineRecord* g_tl_buf = nullptr;
-static uint64_t g_tl_slots = 0, g_tl_per_slot = 0, g_tl_next = 0;
-static TimelineRecord* timeline_next(uint64_t blocks) {
-    if (!g_tl_buf || blocks > g_tl_per_slot) return nullptr;
-    return g_tl_buf + (g_tl_next++ % g_tl_slots) * g_tl_per_slot;
-}
-extern "C" MCCLX_API void mcclx_tune_timeline(void* device_buf, uint64_t slots, uint64_t records_per_slot) {
-    g_tl_buf = static_cast<TimelineRecord*>(device_buf);
-    g_tl_slots = slots;
-    g_tl_per_slot = records_per_slot;
-    g_tl_next = 0;
-}
+// Where the next by-value launches put their records (measurement build): a caller-provided
+// device buffer cut into `slots` regions of `per_slot` records, used round robin.  This file
+// is compiled once per part; part 0 holds the state.
+TimelineRecord* timeline_next(uint64_t blocks);
 #endif
 
 // ------------------------------------------------------ reads, then writes
@@ -795,8 +720,15 @@ template <class C, int T, int HB, bool FAN>
 static bool hold_launch(hipStream_t st, FewArgs& a, uint64_t packets, uint32_t gate, const LaunchParams& lp) {
     const uint32_t cap = hold_capacity<C, T, HB, FAN>(lp.cus);
     if (cap < (uint32_t)a.nseg) return false;
-    const uint32_t hx = cap / (uint32_t)a.nseg;
+    uint32_t hx = cap / (uint32_t)a.nseg;
     if (packets > (uint64_t)hx * HB * T) return false;
+    // As many blocks as the device holds -- the more waves share the launch's loads, the sooner
+    // they are through (C2 with 267 instead of 341 blocks per segment: 16 us instead of 13) --
+    // but a whole number of fours per segment: measured on a 25 MiB bucket of three segments,
+    // 340 and 336 blocks per segment run the launch in 13.07 us, 341 in 13.22, 338 in 13.3 and
+    // 339 in 13.9 (which blocks of the three segments share an XCD, and the distance between a
+    // lane's packets, change with it).
+    if (hx >= 8 && packets <= (uint64_t)(hx & ~3u) * HB * T) hx &= ~3u;
 #if MCCLX_TUNE_TIMELINE
     a.timeline = timeline_next((uint64_t)hx * (uint64_t)a.nseg);
 #endif
@@ -817,15 +749,11 @@ static bool try_hold(hipStream_t st, FewArgs& a, uint64_t maxc, const LaunchPara
     uint64_t ticks = lp.hold_latency_ticks + read_bytes / lp.hold_bytes_per_tick;
     const uint32_t gate = ticks > 100000 ? 100000u : (uint32_t)ticks;  // a millisecond at most
     const uint64_t packets = (maxc + C::E - 1) / C::E;
-#ifdef MCCLX_TUNE_HOLD_256
-    const bool took = hold_launch<C, 4, 256, FAN>(st, a, packets, gate, lp) || hold_launch<C, 5, 256, FAN>(st, a, packets, gate, lp);
-#else
     // A fold with one output takes four packets per lane if that covers it.  One that writes as
     // much as it reads (fan-out) does better with five and fewer waves: the one-launch allreduce
     // of a 25 MiB bucket 26.5 us against 27.6 us (of a 16 MiB bucket 17.4 against 17.2 us).
     const bool took = FAN ? (hold_launch<C, 5, 512, FAN>(st, a, packets, gate, lp) || hold_launch<C, 4, 512, FAN>(st, a, packets, gate, lp))
                           : (hold_launch<C, 4, 512, FAN>(st, a, packets, gate, lp) || hold_launch<C, 5, 512, FAN>(st, a, packets, gate, lp));
-#endif
     if (took && lp.held) *lp.held = true;
     return took;
 }
@@ -901,15 +829,6 @@ constexpr bool kFanPlan = C::OP == MCCLX_SUM && C::ACC == MCCLX_ACC_STEP && C::K
 // ----------------------------------------------------------------- dispatch
 
 
-#ifdef MCCLX_TUNE_MINIMAL
-static size_t wide_lds_bytes() {  // tuning: dynamic LDS reserved per block of a wide fold, to cap blocks per CU
-    static const size_t v = [] { const char* e = getenv("MCCLX_WIDE_LDS"); return e ? (size_t)atol(e) : 0; }();
-    return v;
-}
-#else
-static constexpr size_t wide_lds_bytes() { return 0; }
-#endif
-
 template <class C>
 static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
     const uint64_t span = (uint64_t)C::U * C::BLOCK * C::E;  // elements per block iteration
@@ -958,9 +877,6 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
         // one block per tile of the longest segment (the by-value kernel does not loop)
         uint64_t gx = (maxc + span - 1) / span;
         if (gx >> 31) return hipErrorInvalidValue;
-#if MCCLX_TUNE_XCD
-        gx = (gx + MCCLX_TUNE_XCD - 1) / MCCLX_TUNE_XCD * MCCLX_TUNE_XCD;
-#endif
         if constexpr (kHoldPlan<C>)
             if (try_hold<C, false>(st, a, maxc, lp)) return hipGetLastError();
 #if MCCLX_TUNE_TIMELINE
@@ -969,7 +885,7 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
         if constexpr (kLightPlan<C>)
             fold_few_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(C::BLOCK), 0, st>>>(a);
         else
-            fold_few_wide_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(C::BLOCK), wide_lds_bytes(), st>>>(a);
+            fold_few_wide_kernel<C><<<dim3((uint32_t)gx, (uint32_t)a.nseg), dim3(C::BLOCK), 0, st>>>(a);
     }
     return hipGetLastError();
 }
@@ -982,6 +898,21 @@ static hipError_t launch_cfg(hipStream_t st, const LaunchParams& lp) {
 #define MCCLX_PART -1
 #endif
 #define MCCLX_HAS_PART(n) (MCCLX_PART == -1 || MCCLX_PART == (n))
+
+#if MCCLX_TUNE_TIMELINE && MCCLX_HAS_PART(0)
+static TimelineRecord* g_tl_buf = nullptr;
+static uint64_t g_tl_slots = 0, g_tl_per_slot = 0, g_tl_next = 0;
+TimelineRecord* timeline_next(uint64_t blocks) {
+    if (!g_tl_buf || blocks > g_tl_per_slot) return nullptr;
+    return g_tl_buf + (g_tl_next++ % g_tl_slots) * g_tl_per_slot;
+}
+extern "C" MCCLX_API void mcclx_tune_timeline(void* device_buf, uint64_t slots, uint64_t records_per_slot) {
+    g_tl_buf = static_cast<TimelineRecord*>(device_buf);
+    g_tl_slots = slots;
+    g_tl_per_slot = records_per_slot;
+    g_tl_next = 0;
+}
+#endif
 
 #if MCCLX_HAS_PART(0)
 int plan_block(const PlanKey& key);
@@ -998,13 +929,13 @@ uint32_t items_for(const PlanKey& k, uint64_t count) {
     return (uint32_t)(n ? n : (count ? 1 : 0));
 }
 
-static bool key_is_wide(const PlanKey& key) { return key_pack_elems(key) == 8 && key.k >= MCCLX_TUNE_WIDE_MINK; }
+static bool key_is_wide(const PlanKey& key) { return key_pack_elems(key) == 8 && key.k >= kWideMinK; }
 
 int plan_block(const PlanKey& key) {
     const bool decode = key.k == 1 && key.io == MCCLX_IO_OUT_F32;
     if (key_is_wide(key)) return kWideBlock;
-    if ((key.dtype == MCCLX_F32 && key.k >= 2) || decode) return MCCLX_TUNE_F32_BLOCK;
-    return (key.io == MCCLX_IO_ALL_F32 && key.k >= 2) ? MCCLX_TUNE_ALLF32_BLOCK : kBlock;
+    if ((key.dtype == MCCLX_F32 && key.k >= 2) || decode) return kF32Block;
+    return (key.io == MCCLX_IO_ALL_F32 && key.k >= 2) ? kAllF32Block : kBlock;
 }
 
 bool fan_plan_ok(const PlanKey& key) {
@@ -1013,7 +944,6 @@ bool fan_plan_ok(const PlanKey& key) {
 }
 
 int plan_unroll(const PlanKey& key) {
-    if (MCCLX_TUNE_U) return MCCLX_TUNE_U;
     if (key_is_wide(key)) return kWideU;
     if (key.topo == MCCLX_TOPO_BINOMIAL) return 1;
     return (key_pack_elems(key) == 8 || (key.k == 1 && key.io != MCCLX_IO_PURE)) ? 2 : 1;
@@ -1071,41 +1001,6 @@ hipError_t launch_part_sum_bf16_all_f32(hipStream_t st, const PlanKey& key, cons
 hipError_t launch_part_ops_f32(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
 hipError_t launch_part_ops_f16(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
 hipError_t launch_part_ops_bf16(hipStream_t st, const PlanKey& key, const LaunchParams& lp);
-
-#ifdef MCCLX_TUNE_MINIMAL
-// tuning builds: only the measured configurations, to keep compile times short
-hipError_t launch_fold(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
-    if (key.op == MCCLX_SUM && key.acc == MCCLX_ACC_STEP && key.topo == MCCLX_TOPO_FOLD) {
-        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_OWN_FIRST_F32 && key.k == 3)
-            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_OWN_FIRST_F32, 3, 0, 0, 0>>(st, lp);
-        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_OWN_FIRST_F32 && key.k == 1)
-            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_OWN_FIRST_F32, 1, 0, 0, 0>>(st, lp);
-        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_ALL_F32 && key.k == 3)
-            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_ALL_F32, 3, 0, 0, 0>>(st, lp);
-        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_OWN_LAST_F32 && key.k == 4)
-            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_OWN_LAST_F32, 4, 0, 0, 0>>(st, lp);
-        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_PURE && key.k == 8)
-            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_PURE, 8, 0, 0, 0>>(st, lp);
-        if (key.dtype == MCCLX_F32 && key.k == 3)
-            return launch_cfg<Cfg<MCCLX_F32, MCCLX_IO_PURE, 3, 0, 0, 0>>(st, lp);
-        if (key.dtype == MCCLX_F32 && key.k == 2)
-            return launch_cfg<Cfg<MCCLX_F32, MCCLX_IO_PURE, 2, 0, 0, 0>>(st, lp);
-        if (key.dtype == MCCLX_F32 && key.k == 1)
-            return launch_cfg<Cfg<MCCLX_F32, MCCLX_IO_PURE, 1, 0, 0, 0>>(st, lp);
-        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_OUT_F32 && key.k == 1)
-            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_OUT_F32, 1, 0, 0, 0>>(st, lp);
-        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_PURE && key.k == 2)
-            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_PURE, 2, 0, 0, 0>>(st, lp);
-        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_PURE && key.k == 3)
-            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_PURE, 3, 0, 0, 0>>(st, lp);
-        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_PURE && key.k == 4)
-            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_PURE, 4, 0, 0, 0>>(st, lp);
-        if (key.dtype == MCCLX_BF16 && key.io == MCCLX_IO_PURE && key.k == 1)
-            return launch_cfg<Cfg<MCCLX_BF16, MCCLX_IO_PURE, 1, 0, 0, 0>>(st, lp);
-    }
-    return hipErrorInvalidValue;
-}
-#else
 
 #if MCCLX_HAS_PART(0)
 hipError_t launch_fold(hipStream_t st, const PlanKey& key, const LaunchParams& lp) {
@@ -1174,7 +1069,5 @@ hipError_t launch_part_sum_bf16_all_f32(hipStream_t st, const PlanKey& key, cons
     MCCLX_TOPO_CASES(MCCLX_BF16, MCCLX_IO_ALL_F32, MCCLX_SUM, MCCLX_ACC_F32)
 }
 #endif
-
-#endif  // MCCLX_TUNE_MINIMAL
 
 }  // namespace mcclx

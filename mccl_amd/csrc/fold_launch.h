@@ -12,10 +12,7 @@ namespace mcclx {
 // Segments that travel by value in the kernel arguments (32 x 88 B = 2.8 KB).
 // A block that finds its descriptor there starts loading data at once; one that
 // must first fetch it from a device table loses 5-10 % on large segments.
-#ifndef MCCLX_TUNE_FEW_SEGS
-#define MCCLX_TUNE_FEW_SEGS 32
-#endif
-constexpr int kFewSegs = MCCLX_TUNE_FEW_SEGS;
+constexpr int kFewSegs = 32;
 
 // Device-side view of mcclx_seg (same layout: the table is uploaded verbatim).
 struct SegArgs {

@@ -10,6 +10,7 @@
 #include <cstdlib>
 #include <atomic>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -79,7 +80,8 @@ struct mcclx_ctx {
     uint64_t hold_min_read_bytes = 10ull << 20;
     uint32_t hold_latency_ticks = 40, hold_bytes_per_tick = 71000;  // in ticks of 100 MHz
     uint32_t wall_khz = 100000;                                      // the device's wall clock
-    bool hold_enabled = true;
+    bool hold_measured = false;        // the gate's rate was measured on this device (not the default)
+    std::atomic<bool> hold_enabled{true};  // a completer thread may switch it while ranks launch
     std::atomic<uint64_t> hold_launches{0};
     bool batch_active = false;
     std::string batch_label;
@@ -91,8 +93,6 @@ struct mcclx_ctx {
     std::unordered_map<uint64_t, Ticket> tickets;
     std::vector<hipEvent_t> free_events;
     uint64_t next_ticket = 1;
-    hipEvent_t t0 = nullptr, t1 = nullptr;
-    bool timing = false;
     TableSlot slots[kTableSlots];
     int next_slot = 0;
     std::unordered_map<void*, uint64_t> host_allocs;
@@ -308,8 +308,22 @@ int check_segs(mcclx_ctx* ctx, const mcclx::PlanKey& key, const mcclx_seg* segs,
             if ((uintptr_t)d % (out_f32 ? 4 : 2))
                 return fail(MCCLX_ERR_INVALID, "segment %u: fan-out destination in[%d]=%p is not element aligned", s,
                             key.k + f, d);
-            if (ctx->validate)
+            if (ctx->validate) {
                 if (int rc = check_range(d, g.count * (out_f32 ? 4 : 2), "fan-out destination", s)) return rc;
+                // a destination may BE one of the operands (each lane reads a packet before it
+                // writes it); one that overlaps an operand at another offset would be read by
+                // some lanes after other lanes have written it
+                const char* d0 = static_cast<const char*>(d);
+                const char* d1 = d0 + g.count * (out_f32 ? 4 : 2);
+                for (int i = 0; i < key.k; ++i) {
+                    const char* i0 = static_cast<const char*>(g.in[i]);
+                    const char* i1 = i0 + g.count * (in_is_f32(key, i) ? 4 : 2);
+                    if (d0 != i0 && d0 < i1 && i0 < d1)
+                        return fail(MCCLX_ERR_INVALID,
+                                    "segment %u: fan-out destination in[%d]=%p overlaps operand in[%d]=%p at another offset",
+                                    s, key.k + f, d, i, g.in[i]);
+                }
+            }
         }
         if (ctx->validate) {
             for (int i = 0; i < key.k; ++i)
@@ -408,7 +422,7 @@ int launch_by_value(mcclx_ctx* ctx, const mcclx::PlanKey& key, float scale_f, in
     lp.cus = ctx->cus;
     bool held = false;
     lp.held = &held;
-    lp.hold_min_read_bytes = ctx->hold_enabled ? ctx->hold_min_read_bytes : 0;
+    lp.hold_min_read_bytes = ctx->hold_enabled.load(std::memory_order_relaxed) ? ctx->hold_min_read_bytes : 0;
     lp.hold_latency_ticks = (uint32_t)((uint64_t)ctx->hold_latency_ticks * ctx->wall_khz / 100000);
     lp.hold_bytes_per_tick = (uint32_t)((uint64_t)ctx->hold_bytes_per_tick * 100000 / ctx->wall_khz);
     if (lp.hold_bytes_per_tick == 0) lp.hold_bytes_per_tick = 1;
@@ -426,6 +440,20 @@ int launch_by_value(mcclx_ctx* ctx, const mcclx::PlanKey& key, float scale_f, in
     return MCCLX_OK;
 }
 
+// By value the grid is (tiles of the longest segment) x (segments), so a launch whose
+// segments differ wildly in length would consist mostly of blocks with nothing to do;
+// such a launch takes a table, which has one block per tile.
+bool even_enough(const mcclx::PlanKey& key, const mcclx_seg* segs, uint32_t nseg) {
+    if (nseg <= 4) return true;
+    uint64_t longest = 0, total = 0;
+    for (uint32_t s = 0; s < nseg; ++s) {
+        const uint64_t n = mcclx::items_for(key, segs[s].count);
+        total += n;
+        if (n > longest) longest = n;
+    }
+    return longest * nseg <= 4 * total + 64;
+}
+
 int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uint32_t nseg) {
     if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
     mcclx::PlanKey key;
@@ -439,20 +467,8 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
 
     mcclx::LaunchParams lp;
     lp.max_blocks = ctx->max_blocks;
-    // By value: the grid is (tiles of the longest segment) x (segments), so a launch
-    // whose segments differ wildly in length would consist mostly of blocks with
-    // nothing to do; such a launch takes the table, which has one block per tile.
-    bool by_value = nseg <= ctx->few_max;
-    if (by_value && nseg > 4) {
-        uint64_t longest = 0, total = 0;
-        for (uint32_t s = 0; s < nseg; ++s) {
-            uint64_t n = mcclx::items_for(key, segs[s].count);
-            total += n;
-            if (n > longest) longest = n;
-        }
-        by_value = longest * nseg <= 4 * total + 64;
-    }
-    if (by_value) return launch_by_value(ctx, key, scale_f, has_scale, segs, nseg, fan);
+    if (nseg <= ctx->few_max && even_enough(key, segs, nseg))
+        return launch_by_value(ctx, key, scale_f, has_scale, segs, nseg, fan);
 
     // descriptor table: segs, then nseg+1 work-item prefix sums
     std::lock_guard<std::mutex> lk(ctx->mu);
@@ -503,6 +519,88 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
     return MCCLX_OK;
 }
 
+// The hold form's gate follows the device.  Its model -- no store before
+// latency + bytes read / rate -- has one constant that differs from part to part and from
+// one memory configuration to the next: the rate at which a launch's reads come in.  It is
+// measured once per device and process, when the first context is made: read-only launches of
+// two sizes over a scratch buffer larger than the Infinity Cache (so they read HBM, as a
+// gradient bucket does), the difference of their times over the difference of their sizes.
+// On MI355X the best gate of a 25 MiB bucket, swept, sits at 0.995 of the rate this probe
+// measures (a fold's reads come in a little slower than a single stream's: several address
+// streams, the arithmetic of the late waves), and that ratio is what carries over to
+// another device.
+// MCCLX_HOLD_CALIBRATE=0 keeps the defaults; the MCCLX_HOLD_* knobs override either.
+struct HoldModel {
+    uint32_t latency_ticks = 40;      // ticks of 100 MHz
+    uint32_t bytes_per_tick = 71000;  // per tick of 100 MHz
+    bool measured = false;
+};
+constexpr double kHoldGateRatio = 0.995;
+
+HoldModel measure_hold_model() {  // the device is current
+    HoldModel m;
+    if (const char* v = getenv("MCCLX_HOLD_CALIBRATE"))
+        if (v[0] == '0') return m;
+    constexpr size_t kBig = 48u << 20, kSmall = 24u << 20;
+    constexpr int kCopies = 8;  // 384 MiB: more than the 256 MiB Infinity Cache
+    char* buf = nullptr;
+    hipStream_t st = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    auto cleanup = [&] {
+        if (e0) (void)hipEventDestroy(e0);
+        if (e1) (void)hipEventDestroy(e1);
+        if (st) (void)hipStreamDestroy(st);
+        if (buf) (void)hipFree(buf);
+        (void)hipGetLastError();
+    };
+    if (hipMalloc(reinterpret_cast<void**>(&buf), kBig * kCopies) != hipSuccess ||
+        hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+        cleanup();
+        return m;
+    }
+    bool ok = true;
+    for (int i = 0; i < kCopies && ok; ++i)  // a payload of mixed bits (zero-filled memory reads faster)
+        ok = mcclx::launch_stream_probe(st, buf + (size_t)i * kBig, kBig, true) == hipSuccess;
+    auto timed = [&](size_t nbytes) -> double {  // microseconds per launch, best of three rounds
+        double best = 1e30;
+        for (int round = 0; round < 5 && ok; ++round) {
+            constexpr int kReps = 24;
+            for (int i = 0; i < 4 && ok; ++i)
+                ok = mcclx::launch_stream_probe(st, buf + (size_t)(i % kCopies) * kBig, nbytes, false) == hipSuccess;
+            ok = ok && hipEventRecord(e0, st) == hipSuccess;
+            for (int i = 0; i < kReps && ok; ++i)
+                ok = mcclx::launch_stream_probe(st, buf + (size_t)((i + 4) % kCopies) * kBig, nbytes, false) == hipSuccess;
+            ok = ok && hipEventRecord(e1, st) == hipSuccess && hipEventSynchronize(e1) == hipSuccess;
+            float ms = 0.f;
+            ok = ok && hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+            if (ok && ms * 1e3 / kReps < best) best = ms * 1e3 / kReps;
+        }
+        return best;
+    };
+    const double t_small = timed(kSmall), t_big = timed(kBig);
+    cleanup();
+    if (!ok || !(t_big > t_small)) return m;
+    const double probe_rate = (double)(kBig - kSmall) / ((t_big - t_small) * 100.0);  // bytes per 10 ns
+    const double rate = probe_rate * kHoldGateRatio;
+    // a device busy with someone else's work while this ran gives nonsense: keep the default then
+    if (rate < 0.5 * m.bytes_per_tick || rate > 2.0 * m.bytes_per_tick) return m;
+    m.bytes_per_tick = (uint32_t)rate;
+    m.measured = true;
+    return m;
+}
+
+HoldModel device_hold_model(int device) {  // `device` is current
+    static std::mutex mu;
+    static std::map<int, HoldModel> cache;
+    std::lock_guard<std::mutex> lk(mu);
+    auto it = cache.find(device);
+    if (it != cache.end()) return it->second;
+    const HoldModel m = measure_hold_model();
+    cache[device] = m;
+    return m;
+}
+
 int make_ctx(int device, hipStream_t borrowed, bool borrow, mcclx_ctx** out) {
     if (!out) return fail(MCCLX_ERR_INVALID, "out is null");
     *out = nullptr;
@@ -543,8 +641,14 @@ int make_ctx(int device, hipStream_t borrowed, bool borrow, mcclx_ctx** out) {
         if (x >= 0 && x <= mcclx::kFewSegs) ctx->few_max = (uint32_t)x;
     }
     if (const char* v = getenv("MCCLX_VALIDATE")) ctx->validate = (v[0] == '1');
+    {
+        const HoldModel hm = device_hold_model(device);
+        ctx->hold_latency_ticks = hm.latency_ticks;
+        ctx->hold_bytes_per_tick = hm.bytes_per_tick;
+        ctx->hold_measured = hm.measured;
+    }
     // MCCLX_HOLD=0 switches the reads-then-writes launches off; the other three are tuning knobs
-    if (const char* v = getenv("MCCLX_HOLD")) ctx->hold_enabled = v[0] != '0';
+    if (const char* v = getenv("MCCLX_HOLD")) ctx->hold_enabled.store(v[0] != '0');
     if (const char* v = getenv("MCCLX_HOLD_MIN_BYTES")) {
         const unsigned long long x = strtoull(v, nullptr, 10);
         ctx->hold_min_read_bytes = x ? x : 1;
@@ -552,7 +656,10 @@ int make_ctx(int device, hipStream_t borrowed, bool borrow, mcclx_ctx** out) {
     if (const char* v = getenv("MCCLX_HOLD_LATENCY_TICKS")) ctx->hold_latency_ticks = (uint32_t)strtoul(v, nullptr, 10);
     if (const char* v = getenv("MCCLX_HOLD_BYTES_PER_TICK")) {
         const unsigned long x = strtoul(v, nullptr, 10);
-        if (x >= 1000 && x <= 1000000) ctx->hold_bytes_per_tick = (uint32_t)x;
+        if (x >= 1000 && x <= 1000000) {
+            ctx->hold_bytes_per_tick = (uint32_t)x;
+            ctx->hold_measured = false;
+        }
     }
     e = mcclx::static_table_resolve(device, &ctx->static_table);  // `device` is current (guard above)
     if (e != hipSuccess) {
@@ -572,6 +679,21 @@ int make_ctx(int device, hipStream_t borrowed, bool borrow, mcclx_ctx** out) {
     *out = ctx;
     return MCCLX_OK;
 }
+
+// Host-side guard of a GPU's static descriptor table: held for the duration of one
+// allocation-free call.
+constexpr int kMaxGuardedDevices = 64;
+std::atomic<bool> g_static_table_busy[kMaxGuardedDevices];
+struct StaticTableUse {
+    int dev;
+    bool mine;
+    explicit StaticTableUse(int device) : dev(device), mine(true) {
+        if (dev >= 0 && dev < kMaxGuardedDevices) mine = !g_static_table_busy[dev].exchange(true, std::memory_order_acquire);
+    }
+    ~StaticTableUse() {
+        if (mine && dev >= 0 && dev < kMaxGuardedDevices) g_static_table_busy[dev].store(false, std::memory_order_release);
+    }
+};
 
 int get_event(mcclx_ctx* ctx, hipEvent_t* ev) {
     if (!ctx->free_events.empty()) {
@@ -604,8 +726,6 @@ int mcclx_destroy(mcclx_ctx* ctx) {
     for (auto ev : ctx->free_events) (void)hipEventDestroy(ev);
     for (auto ev : ctx->xev)
         if (ev) (void)hipEventDestroy(ev);
-    if (ctx->t0) (void)hipEventDestroy(ctx->t0);
-    if (ctx->t1) (void)hipEventDestroy(ctx->t1);
     for (auto& sl : ctx->slots) {
         if (sl.host) (void)hipHostFree(sl.host);
         if (sl.dev) (void)hipFree(sl.dev);
@@ -627,9 +747,15 @@ void* mcclx_queue_stream(mcclx_ctx* ctx) { return ctx ? (void*)ctx->stream : nul
 int mcclx_device_cus(mcclx_ctx* ctx) { return ctx ? ctx->cus : 0; }
 uint64_t mcclx_launch_count(mcclx_ctx* ctx) { return ctx ? ctx->launches.load() : 0; }
 uint64_t mcclx_hold_launch_count(mcclx_ctx* ctx) { return ctx ? ctx->hold_launches.load() : 0; }
+int mcclx_hold_model(mcclx_ctx* ctx, uint32_t* latency_ticks, uint32_t* bytes_per_tick) {
+    if (!ctx) return 0;
+    if (latency_ticks) *latency_ticks = ctx->hold_latency_ticks;
+    if (bytes_per_tick) *bytes_per_tick = ctx->hold_bytes_per_tick;
+    return ctx->hold_measured ? 1 : 0;
+}
 int mcclx_set_hold(mcclx_ctx* ctx, int enabled) {
     if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
-    ctx->hold_enabled = enabled != 0;
+    ctx->hold_enabled.store(enabled != 0, std::memory_order_relaxed);
     return MCCLX_OK;
 }
 
@@ -655,7 +781,17 @@ int mcclx_fold_batched_noalloc(mcclx_ctx* ctx, const mcclx_plan* plan, const mcc
     if (nseg == 0) return MCCLX_OK;
     DeviceGuard guard(ctx->device);
     if (!guard.ok) return fail(MCCLX_ERR_HIP, "hipSetDevice(%d) failed", ctx->device);
-    if (nseg <= (uint32_t)mcclx::kFewSegs) return launch_by_value(ctx, key, scale_f, has_scale, segs, nseg, fan);
+    if (nseg <= (uint32_t)mcclx::kFewSegs && even_enough(key, segs, nseg))
+        return launch_by_value(ctx, key, scale_f, has_scale, segs, nseg, fan);
+
+    // One table per GPU, shared by every context on it: a second call that enters while this
+    // one is still writing its descriptors would mix the two tables.  (Calls on one context
+    // are ordered by its queue; launches of different contexts that are both already queued
+    // and overlap on the device still race -- the host cannot see that.)
+    StaticTableUse use(ctx->device);
+    if (!use.mine)
+        return fail(MCCLX_ERR_STATE,
+                    "fold_batched_noalloc: another call is filling GPU %d's static descriptor table", ctx->device);
 
     uint64_t total = 0, uniform = mcclx::items_for(key, segs[0].count);
     for (uint32_t s = 0; s < nseg; ++s) {
@@ -779,19 +915,6 @@ int mcclx_copy(mcclx_ctx* ctx, void* dst, const void* src, uint64_t nbytes) {
     DeviceGuard guard(ctx->device);
     hipError_t e = mcclx::launch_copy(ctx->stream, dst, src, nbytes, ctx->max_blocks);
     if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "copy launch failed: %s", hipGetErrorString(e));
-    ++ctx->launches;
-    return MCCLX_OK;
-}
-
-int mcclx_probe_stream(mcclx_ctx* ctx, void* buf, uint64_t nbytes, int write) {
-    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
-    if (nbytes == 0) return MCCLX_OK;
-    if (!buf || (uintptr_t)buf % 4) return fail(MCCLX_ERR_INVALID, "probe_stream: buffer is null or not 4-byte aligned");
-    if (ctx->validate)
-        if (int rc = check_range(buf, nbytes, "buf", 0)) return rc;
-    DeviceGuard guard(ctx->device);
-    hipError_t e = mcclx::launch_stream_probe(ctx->stream, buf, nbytes, write != 0);
-    if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "probe launch failed: %s", hipGetErrorString(e));
     ++ctx->launches;
     return MCCLX_OK;
 }
@@ -1006,30 +1129,6 @@ int mcclx_event_wait(mcclx_ctx* ctx, uint64_t ticket) {
     return MCCLX_OK;
 }
 
-int mcclx_timer_begin(mcclx_ctx* ctx) {
-    if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
-    REFUSE_WHILE_RECORDING(ctx, "timer_begin");
-    DeviceGuard guard(ctx->device);
-    if (!ctx->t0) {
-        HIP_TRY(hipEventCreate(&ctx->t0));
-        HIP_TRY(hipEventCreate(&ctx->t1));
-    }
-    HIP_TRY(hipEventRecord(ctx->t0, ctx->stream));
-    ctx->timing = true;
-    return MCCLX_OK;
-}
-
-int mcclx_timer_end(mcclx_ctx* ctx, float* elapsed_ms) {
-    if (!ctx || !elapsed_ms) return fail(MCCLX_ERR_INVALID, "timer_end: null argument");
-    if (!ctx->timing) return fail(MCCLX_ERR_STATE, "timer_end without timer_begin");
-    DeviceGuard guard(ctx->device);
-    HIP_TRY(hipEventRecord(ctx->t1, ctx->stream));
-    HIP_TRY(hipEventSynchronize(ctx->t1));
-    HIP_TRY(hipEventElapsedTime(elapsed_ms, ctx->t0, ctx->t1));
-    ctx->timing = false;
-    return MCCLX_OK;
-}
-
 int mcclx_graph_begin(mcclx_ctx* ctx) {
     if (!ctx) return fail(MCCLX_ERR_STATE, "context is null (mcclx_init not called)");
     if (ctx->capturing) return fail(MCCLX_ERR_STATE, "graph recording already active");
@@ -1209,5 +1308,17 @@ int mcclx_host_free(mcclx_ctx* ctx, void* host_ptr) {
     HIP_TRY(hipHostFree(host_ptr));
     return MCCLX_OK;
 }
+
+#if MCCLX_TUNE_TIMELINE
+// Measurement build only (include/mcclx_bench.h): one launch that only reads or only
+// writes `nbytes` of `buf` on `hip_stream`, with the copy kernel's access shape.
+MCCLX_API int mcclx_bench_probe(void* hip_stream, void* buf, uint64_t nbytes, int write) {
+    if (nbytes == 0) return MCCLX_OK;
+    if (!buf || (uintptr_t)buf % 4) return fail(MCCLX_ERR_INVALID, "bench_probe: buffer is null or not 4-byte aligned");
+    hipError_t e = mcclx::launch_stream_probe(static_cast<hipStream_t>(hip_stream), buf, nbytes, write != 0);
+    if (e != hipSuccess) return fail(MCCLX_ERR_HIP, "probe launch failed: %s", hipGetErrorString(e));
+    return MCCLX_OK;
+}
+#endif
 
 }  // extern "C"

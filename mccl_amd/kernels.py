@@ -128,13 +128,23 @@ class ReduceQueue:
     def wait(self, ticket: int) -> None:
         L.check(L.lib().mcclx_event_wait(self.handle, ticket))
 
+    # Device time on the queue, for measurement: torch events recorded on the queue's own
+    # stream (torch.cuda.Event sees the stream it is recorded on, not the current one).
+    def _torch_stream(self) -> "torch.cuda.Stream":
+        if getattr(self, "_ext_stream", None) is None:
+            self._ext_stream = torch.cuda.ExternalStream(self.stream, device=self.device)
+        return self._ext_stream
+
     def timer_begin(self) -> None:
-        L.check(L.lib().mcclx_timer_begin(self.handle))
+        self._t0 = torch.cuda.Event(enable_timing=True)
+        self._t1 = torch.cuda.Event(enable_timing=True)
+        self._t0.record(self._torch_stream())
 
     def timer_end(self) -> float:
-        ms = C.c_float()
-        L.check(L.lib().mcclx_timer_end(self.handle, C.byref(ms)))
-        return ms.value
+        """Milliseconds between timer_begin and now, both on the queue; waits for the queue."""
+        self._t1.record(self._torch_stream())
+        self._t1.synchronize()
+        return self._t0.elapsed_time(self._t1)
 
     # -- launch graphs --------------------------------------------------------
     def graph_begin(self) -> None:
@@ -195,9 +205,21 @@ class ReduceQueue:
     def copy(self, dst_ptr: int, src_ptr: int, nbytes: int) -> None:
         L.check(L.lib().mcclx_copy(self.handle, C.c_void_p(dst_ptr), C.c_void_p(src_ptr), nbytes))
 
+    def hold_model(self):
+        """(latency_ticks, bytes_per_tick, measured): the gate of the hold form on this device."""
+        lat, bpt = C.c_uint32(), C.c_uint32()
+        measured = L.lib().mcclx_hold_model(self.handle, C.byref(lat), C.byref(bpt))
+        return lat.value, bpt.value, bool(measured)
+
     def probe_stream(self, ptr: int, nbytes: int, write: bool) -> None:
-        """One read-only or write-only pass over a buffer (measurement aid)."""
-        L.check(L.lib().mcclx_probe_stream(self.handle, C.c_void_p(ptr), nbytes, int(write)))
+        """One read-only or write-only pass over a buffer on this queue: a launch of the
+        measurement build (python -m mccl_amd.build --bench), which must be there."""
+        B = L.bench_lib()
+        if B is None:
+            raise MCCLError("[MCCL] the measurement build is missing: python -m mccl_amd.build --bench", L.ERR_STATE)
+        rc = B.mcclx_bench_probe(C.c_void_p(self.stream), C.c_void_p(ptr), nbytes, int(write))
+        if rc != L.OK:
+            raise MCCLError(B.mcclx_last_error().decode("utf-8", "replace"), rc)
 
     def copy_batched(self, triples) -> None:
         """Many (dst, src, nbytes) copies in one launch (a few large ones go out one by one)."""

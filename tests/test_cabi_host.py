@@ -34,7 +34,19 @@ def test_header_symbols_are_all_exported_and_bound(L):
         assert hasattr(raw, n), f"{n} declared in mcclx.h but not exported"
         assert n in L.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(L.SIGNATURES) == names
-    assert L.lib().mcclx_abi_version() == 3
+    assert L.lib().mcclx_abi_version() == 4
+
+
+def test_measurement_aids_are_not_in_the_shipped_library(L):
+    """The probe launch, the event timer and the per-block timeline belong to the measurement
+    build (include/mcclx_bench.h); libmcclx.so exports nothing that the header does not declare."""
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", L.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = sorted(line.split()[-1] for line in out.splitlines() if " T " in line and "mcclx_" in line.split()[-1])
+    assert exported == declared_symbols() + ([] if "mcclx_fail" in declared_symbols() else ["mcclx_fail"]) or \
+        sorted(set(exported) - {"mcclx_fail"}) == declared_symbols(), sorted(set(exported) ^ set(declared_symbols()))
+    for gone in ("mcclx_probe_stream", "mcclx_timer_begin", "mcclx_timer_end", "mcclx_tune_timeline", "mcclx_bench_probe"):
+        assert gone not in exported
 
 
 def test_struct_layouts_match_header(L):
