@@ -1,22 +1,51 @@
 #include "backend/HostWire.hpp"
 
-#include <c10/hip/HIPStream.h>
+#ifndef MCCL_NULL_DEVICE
 #include <hip/hip_runtime_api.h>
+#endif
 
 #include <algorithm>
 #include <cstring>
 
+#include "backend/Device.hpp"
 #include "backend/Errors.hpp"
 #include "backend/Logging.hpp"
 
 namespace mccl {
 
-struct HostWire::Ctx {
-    mcclx_ctx* ctx = nullptr;
-    hipEvent_t t0 = nullptr, t1 = nullptr;  // device-time bracket around the fold, for the statistics
-    ~Ctx() {
+// Device-time bracket around the fold launch, for the statistics.
+#ifndef MCCL_NULL_DEVICE
+struct FoldTimer {
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    ~FoldTimer() {
         if (t0) (void)hipEventDestroy(t0);
         if (t1) (void)hipEventDestroy(t1);
+    }
+    void begin(void* stream) {
+        if (!t0)
+            MCCL_CHECK(hipEventCreate(&t0) == hipSuccess && hipEventCreate(&t1) == hipSuccess,
+                       "host wire: hipEventCreate failed");
+        MCCL_CHECK(hipEventRecord(t0, static_cast<hipStream_t>(stream)) == hipSuccess, "host wire: hipEventRecord failed");
+    }
+    double end_ms(void* stream) {
+        float ms = 0.f;
+        MCCL_CHECK(hipEventRecord(t1, static_cast<hipStream_t>(stream)) == hipSuccess &&
+                       hipEventSynchronize(t1) == hipSuccess && hipEventElapsedTime(&ms, t0, t1) == hipSuccess,
+                   "host wire: timing the fold failed");
+        return ms;
+    }
+};
+#else
+struct FoldTimer {
+    void begin(void*) {}
+    double end_ms(void*) { return 0.0; }
+};
+#endif
+
+struct HostWire::Ctx {
+    mcclx_ctx* ctx = nullptr;
+    FoldTimer timer;
+    ~Ctx() {
         if (ctx) mcclx_destroy(ctx);
     }
 };
@@ -107,9 +136,8 @@ std::shared_ptr<HostWire::Pinned> HostWire::pinned(std::shared_ptr<Pinned>& slot
 void* HostWire::device_scratch(at::Tensor& slot, uint64_t nbytes) {
     if (!slot.defined() || static_cast<uint64_t>(slot.numel()) < nbytes + 256) {
         check_rc(mcclx_queue_drain(ctx_->ctx));
-        slot = at::empty({static_cast<int64_t>(nbytes + 256)}, at::TensorOptions().dtype(at::kByte).device(at::kCUDA, device_));
-        check_rc(mcclx_queue_wait_stream(
-            ctx_->ctx, static_cast<void*>(c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(device_)).stream())));
+        slot = dev::empty_bytes(static_cast<int64_t>(nbytes + 256), device_);
+        check_rc(mcclx_queue_wait_stream(ctx_->ctx, dev::current_stream(device_)));
     }
     auto p = reinterpret_cast<uintptr_t>(slot.data_ptr());
     return reinterpret_cast<void*>((p + 255) / 256 * 256);
@@ -249,18 +277,9 @@ void HostWire::allreduce(void* tensor, int dtype, uint64_t numel, int op, int al
             s.out = at(tensor, mine->start * ts);
             if (codec) s.wire_out = at(send_dev, mine->start * 2);  // the reduced chunk as it travels on
         }
-        hipStream_t qs = static_cast<hipStream_t>(mcclx_queue_stream(ctx));
-        if (!ctx_->t0) {
-            MCCL_CHECK(hipEventCreate(&ctx_->t0) == hipSuccess && hipEventCreate(&ctx_->t1) == hipSuccess,
-                       "host wire: hipEventCreate failed");
-        }
-        MCCL_CHECK(hipEventRecord(ctx_->t0, qs) == hipSuccess, "host wire: hipEventRecord failed");
+        ctx_->timer.begin(mcclx_queue_stream(ctx));
         check_rc(mcclx_fold_batched(ctx, &plan, &s, 1));
-        float ms = 0.f;
-        MCCL_CHECK(hipEventRecord(ctx_->t1, qs) == hipSuccess && hipEventSynchronize(ctx_->t1) == hipSuccess &&
-                       hipEventElapsedTime(&ms, ctx_->t0, ctx_->t1) == hipSuccess,
-                   "host wire: timing the fold failed");
-        stats_.fold_ms = ms;
+        stats_.fold_ms = ctx_->timer.end_ms(mcclx_queue_stream(ctx));
         stats_.fold_elems = mine->count;
         stats_.fold_peer_bytes = static_cast<uint64_t>(N - 1) * mine->count * es;
         stats_.fold_hbm_bytes = mine->count * ((all_on_wire ? 0 : 2 * ts));

@@ -1,8 +1,5 @@
 #include "backend/ProcessGroupMCCL.hpp"
 
-#include <c10/hip/HIPFunctions.h>
-#include <c10/hip/HIPStream.h>
-
 #include <algorithm>
 #include <atomic>
 #include <condition_variable>
@@ -14,6 +11,7 @@
 #include <mutex>
 #include <tuple>
 
+#include "backend/Device.hpp"
 #include "backend/Errors.hpp"
 #include "backend/HostWire.hpp"
 #include "backend/LocalMesh.hpp"
@@ -37,7 +35,7 @@ c10::intrusive_ptr<c10d::Work> make_completed(c10d::OpType op, std::vector<at::T
 
 // check_mps_ (ProcessGroupMCCL.cpp:72-79) for ROCm tensors.
 void check_gpu_(const at::Tensor& t, const char* op) {
-    MCCL_CHECK(t.is_cuda(), std::string(op) + ": MCCL on MI355X is GPU-only; got " +
+    MCCL_CHECK(dev::on_device(t), std::string(op) + ": MCCL on MI355X is GPU-only; got " +
                                 std::string(c10::DeviceTypeName(t.device().type())) + " tensor");
     MCCL_CHECK(t.is_contiguous(), std::string(op) + ": tensor must be contiguous");
 }
@@ -81,15 +79,14 @@ namespace {
 // stream); the reduce queue is another stream, so it waits for that one before
 // it touches a fresh block.
 void order_after_allocator(mcclx_ctx* ctx, int device) {
-    check_rc(mcclx_queue_wait_stream(
-        ctx, static_cast<void*>(c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(device)).stream())));
+    check_rc(mcclx_queue_wait_stream(ctx, dev::current_stream(device)));
 }
 }  // namespace
 
 // One reduce queue and one grow-only scratch buffer per mesh (per group of
 // ranks sharing the GPU).  The scratch replaces the reference's per-call
 // at::empty recv buffers (ProcessGroupMCCL.cpp:152-162).
-struct ProcessGroupMCCL::Shared {
+struct ProcessGroupMCCL::Shared : std::enable_shared_from_this<ProcessGroupMCCL::Shared> {
     mcclx_ctx* ctx = nullptr;
     at::Tensor scratch;
     int device = 0;
@@ -223,8 +220,7 @@ struct ProcessGroupMCCL::Shared {
                 return t;
             }
         }
-        at::Tensor t = at::empty({static_cast<int64_t>(nbytes)},
-                                 at::TensorOptions().dtype(at::kByte).device(at::kCUDA, device));
+        at::Tensor t = dev::empty_bytes(static_cast<int64_t>(nbytes), device);
         order_after_allocator(on, device);
         return t;
     }
@@ -290,7 +286,14 @@ struct ProcessGroupMCCL::Shared {
         async_buckets += buckets.size();
         if (!completer) completer = std::make_unique<Progress>();
         mcclx_ctx* c = queue(q);
-        completer->submit([this, c, q, id, ticket, buckets = std::move(buckets)]() mutable {
+        // The task keeps this object alive while it runs: settling a Work runs the callbacks of
+        // its Future, and one of them may drop the last process group of the mesh.  The object
+        // then goes when the task's captures do, with nothing of it in use up the stack (its
+        // destructor shuts the completer down from the completer's own thread, which the engine
+        // allows).  From the destructor itself there is no owner left to share with: it waits
+        // for these tasks before it goes on.
+        std::shared_ptr<Shared> self = weak_from_this().lock();
+        completer->submit([this, self, c, q, id, ticket, buckets = std::move(buckets)]() mutable {
             std::exception_ptr failure;
             try {
                 check_rc(mcclx_event_wait(c, ticket));
@@ -388,8 +391,7 @@ struct ProcessGroupMCCL::Shared {
         if (!scratch.defined() || static_cast<uint64_t>(scratch.numel()) < nbytes + 256) {
             check_rc(mcclx_queue_drain(ctx));  // nothing may still read the old buffer
             drop_graphs();                     // recorded launches point into it
-            scratch = at::empty({static_cast<int64_t>(nbytes + 256)},
-                                at::TensorOptions().dtype(at::kByte).device(at::kCUDA, device));
+            scratch = dev::empty_bytes(static_cast<int64_t>(nbytes + 256), device);
             order_after_allocator(ctx, device);
         }
         auto p = reinterpret_cast<uintptr_t>(scratch.data_ptr());
@@ -461,7 +463,7 @@ ProcessGroupMCCL::ProcessGroupMCCL(c10::intrusive_ptr<c10d::Store> store, int ra
     : c10d::Backend(rank, size), store_(std::move(store)), opts_(opts) {
     MCCL_CHECK(rank >= 0 && rank < size, "rank/size invalid");
     try {
-        device_ = static_cast<int>(c10::hip::current_device());
+        device_ = dev::current_device();
     } catch (const std::exception& e) {
         // the reference fails in metal_kernels_init() when there is no Metal device
         throw MCCLError(std::string("no usable GPU for the mccl backend: ") + e.what());
@@ -508,11 +510,18 @@ ProcessGroupMCCL::ProcessGroupMCCL(c10::intrusive_ptr<c10d::Store> store, int ra
 }
 
 ProcessGroupMCCL::~ProcessGroupMCCL() {
+    // (shutdown runs what is queued; called on the engine's own thread -- a callback there
+    // dropped the last reference to this group -- it does so in place instead of joining)
     if (engine_) engine_->shutdown();
     host_wire_.reset();
     mesh_.reset();
     shared_.reset();
-    if (!mesh_key_.empty()) LocalMesh::forget(mesh_key_);
+    if (!mesh_key_.empty()) {
+        LocalMesh::forget(mesh_key_);
+        std::lock_guard<std::mutex> lk(g_shared_mu);
+        auto it = g_shared.find(mesh_key_);
+        if (it != g_shared.end() && it->second.expired()) g_shared.erase(it);  // the last rank of the mesh
+    }
 }
 
 uint64_t ProcessGroupMCCL::graphHits() const { return shared_ ? shared_->graph_hits : 0; }
@@ -537,7 +546,7 @@ std::vector<double> ProcessGroupMCCL::wireStats() const {
 }
 
 void* ProcessGroupMCCL::my_stream() const {
-    return static_cast<void*>(c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(device_)).stream());
+    return dev::current_stream(device_);
 }
 
 void ProcessGroupMCCL::meet(Contribution c, const LocalMesh::Leader& leader) {
@@ -598,10 +607,15 @@ c10::intrusive_ptr<c10d::Work> async_submit_(Progress& engine, mcclx_ctx* ctx, v
         return work;
     }
     work->setSyncCallback([ctx] { check_rc(mcclx_queue_drain(ctx)); });
-    engine.submit([work, title, body = std::move(body)]() mutable {
+    engine.submit([work, ctx, title, body = std::move(body)]() mutable {
         try {
             body();
-            body = nullptr;  // release the captured tensors before anyone is told the work is done
+            // The captured tensors go back before anyone is told the work is done -- but not
+            // before the device has finished with them: a block freed here belongs to the
+            // stream it was allocated on, the launches ran on the reduce queue, and torch's
+            // allocator would hand the block to the next request on that stream at once.
+            check_rc(mcclx_queue_drain(ctx));
+            body = nullptr;
             work->finish();
         } catch (...) {
             body = nullptr;
@@ -838,9 +852,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
                     auto b = weak.lock();
                     if (!b) return;   // settled and released: nothing left to order against
                     if (!b->launched) sh->flush_parked(b->queue);
-                    check_rc(mcclx_stream_wait_queue(
-                        sh->queue(b->queue),
-                        static_cast<void*>(c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(device)).stream())));
+                    check_rc(mcclx_stream_wait_queue(sh->queue(b->queue), dev::current_stream(device)));
                 });
             shared->submit_bucket(bucket);
             return;
@@ -1257,9 +1269,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::send(std::vector<at::Tensor>& t
             p.tag = static_cast<int32_t>(tag);
             p.nbytes = static_cast<uint64_t>(t.nbytes());
             if (p.nbytes) {
-                auto hold = std::make_shared<at::Tensor>(
-                    at::empty({static_cast<int64_t>(p.nbytes)},
-                              at::TensorOptions().dtype(at::kByte).device(at::kCUDA, shared->device)));
+                auto hold = std::make_shared<at::Tensor>(dev::empty_bytes(static_cast<int64_t>(p.nbytes), shared->device));
                 order_after_allocator(shared->ctx, shared->device);
                 check_rc(mcclx_copy(shared->ctx, hold->data_ptr(), t.data_ptr(), p.nbytes));
                 p.data = hold->data_ptr();

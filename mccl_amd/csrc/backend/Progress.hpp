@@ -6,11 +6,21 @@
 // its tests/internal/test_progress.cpp: FIFO order, the destructor drains the
 // queue, shutdown is idempotent, a throwing task does not stop the engine,
 // submit never waits for a running task.
+//
+// One thing the reference leaves open is settled here: the engine may be shut
+// down, or destroyed, from its own worker thread -- by a task (or a callback a
+// task runs) that drops the last reference to whatever owns the engine.  A
+// thread cannot join itself (std::thread::join throws, and a throw inside a
+// destructor ends the process), so in that case shutdown() runs what is still
+// queued right there, on the worker, and lets the thread go; the state the
+// worker loop still needs afterwards is shared with it and outlives the engine,
+// and the end of the process waits for every worker that is still running.
 #pragma once
 
 #include <condition_variable>
 #include <deque>
 #include <functional>
+#include <memory>
 #include <mutex>
 #include <thread>
 
@@ -52,22 +62,33 @@ public:
 
     // Enqueue; returns at once.  Tasks submitted after shutdown() are dropped.
     void submit(Task task);
-    // Run everything already queued, then stop the worker.  Safe to call twice.
+    // Run everything already queued, then stop the worker.  Safe to call twice,
+    // and from the worker thread itself (see above).
     void shutdown();
     // Tasks run so far (for tests and diagnostics).
     size_t completed() const;
     // True when every task submitted so far has run to its end.
     bool idle() const;
+    // True on the engine's own worker thread.
+    bool on_worker_thread() const;
 
 private:
-    void worker();
+    // Everything the worker loop touches: shared with the thread, so that it stays
+    // valid when the engine object is destroyed from inside one of its own tasks.
+    struct State {
+        std::mutex mu;
+        std::condition_variable wake;
+        std::deque<Task> queue;
+        bool closing = false;
+        size_t completed = 0;
+        size_t submitted = 0;
+    };
+    static void worker(std::shared_ptr<State> st);
+    // Takes the next task off the queue (the lock is held on entry and on return), runs it
+    // and destroys it -- captures included -- with every exception contained.
+    static void run_next(State& st, std::unique_lock<std::mutex>& lk);
 
-    mutable std::mutex mu_;
-    std::condition_variable wake_;
-    std::deque<Task> queue_;
-    bool closing_ = false;
-    size_t completed_ = 0;
-    size_t submitted_ = 0;
+    std::shared_ptr<State> st_;
     std::thread thread_;
 };
 

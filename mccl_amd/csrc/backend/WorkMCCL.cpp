@@ -66,7 +66,13 @@ bool WorkMCCL::wait(std::chrono::milliseconds timeout) {
             if (state_ == State::Failed) std::rethrow_exception(error_);
         }
         on_wait_();  // stream-ordered: the caller's stream now waits for the result on the device
-        std::lock_guard<std::mutex> lk(mu_);
+        std::unique_lock<std::mutex> lk(mu_);
+        if (timeout != kNoTimeout) {
+            // A caller that names a timeout asks for the reference's contract (host-blocking,
+            // false when the time is up, WorkMCCL.cpp:51-55): wait until the Work has settled.
+            const auto settled = [this] { return state_ != State::Pending; };
+            if (!settled_cv_.wait_for(lk, timeout, settled)) return false;
+        }
         if (state_ == State::Failed) std::rethrow_exception(error_);
         return true;
     }

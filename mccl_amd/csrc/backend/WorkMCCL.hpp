@@ -36,7 +36,9 @@ public:
     // on the device, for the reduce queue -- and returns; the Work and its Future
     // settle later, when the device has finished.  A Work that has settled by the
     // time of the wait needs no hook (the device work is known to be over); one that
-    // has failed rethrows from wait().
+    // has failed rethrows from wait().  wait(timeout) with a timeout keeps the
+    // reference's contract on top of that: it blocks the host until the Work has
+    // settled and returns false when the time is up first.
     void setWaitHook(std::function<void()> on_wait) { on_wait_ = std::move(on_wait); }
     void finish();
     void finishWithException(std::exception_ptr error);

@@ -17,8 +17,12 @@
 #include <torch/csrc/distributed/c10d/Store.hpp>
 
 #include <execinfo.h>
+#include <fcntl.h>
 #include <signal.h>
 #include <unistd.h>
+
+#include <cstring>
+#include <exception>
 
 #include <atomic>
 #include <chrono>
@@ -46,17 +50,23 @@ void gil_take_back(void* token) {
     if (token) PyEval_RestoreThread(static_cast<PyThreadState*>(token));
 }
 
-// MCCL_ABORT_BACKTRACE=1: when the process aborts, the native stack of the aborting
-// thread goes to stderr before the handler that was installed before runs (Python's
-// faulthandler prints the interpreter's side).  An abort raised by a library on one
-// of the backend's worker threads is otherwise anonymous.
+// MCCL_ABORT_BACKTRACE: when the process aborts, the native stack of the aborting thread is
+// written out before the handler that was installed before runs (Python's faulthandler prints
+// the interpreter's side), and an uncaught C++ exception is named before it ends the process.
+// An abort raised on one of the backend's worker threads is otherwise anonymous.  The value
+// is "1" for stderr or the path of a file to append to -- under a test runner that captures
+// file descriptor 2, what goes to stderr dies with the process, a file does not.
 struct sigaction g_previous_abort_action;
+int g_abort_fd = 2;
+std::terminate_handler g_previous_terminate = nullptr;
+
+void write_all(int fd, const char* text) { (void)!write(fd, text, strlen(text)); }
+
 void abort_backtrace(int sig, siginfo_t* info, void* uctx) {
-    static const char head[] = "\n[MCCL] SIGABRT: native stack of the aborting thread\n";
-    (void)!write(2, head, sizeof head - 1);
+    write_all(g_abort_fd, "\n[MCCL] SIGABRT: native stack of the aborting thread\n");
     void* frames[64];
     const int n = backtrace(frames, 64);
-    backtrace_symbols_fd(frames, n, 2);
+    backtrace_symbols_fd(frames, n, g_abort_fd);
     sigaction(SIGABRT, &g_previous_abort_action, nullptr);
     if (g_previous_abort_action.sa_flags & SA_SIGINFO) {
         if (g_previous_abort_action.sa_sigaction) g_previous_abort_action.sa_sigaction(sig, info, uctx);
@@ -65,9 +75,35 @@ void abort_backtrace(int sig, siginfo_t* info, void* uctx) {
     }
     raise(sig);
 }
+
+// std::terminate: say which exception it was (and that there was none, if so) where the
+// abort handler's stack will follow, then go on to whoever was installed before (abort).
+void terminate_with_message() {
+    write_all(g_abort_fd, "\n[MCCL] std::terminate called");
+    if (std::exception_ptr e = std::current_exception()) {
+        try {
+            std::rethrow_exception(e);
+        } catch (const std::exception& ex) {
+            write_all(g_abort_fd, " with an uncaught exception: ");
+            write_all(g_abort_fd, ex.what());
+        } catch (...) {
+            write_all(g_abort_fd, " with an uncaught exception of a non-standard type");
+        }
+    } else {
+        write_all(g_abort_fd, " without an active exception (a joinable std::thread destroyed, or a throw from a noexcept function)");
+    }
+    write_all(g_abort_fd, "\n");
+    if (g_previous_terminate) g_previous_terminate();
+    abort();
+}
+
 void install_abort_backtrace() {
     const char* e = std::getenv("MCCL_ABORT_BACKTRACE");
-    if (!e || e[0] != '1') return;
+    if (!e || !*e || (e[0] == '0' && !e[1])) return;
+    if (!(e[0] == '1' && !e[1])) {
+        const int fd = open(e, O_WRONLY | O_CREAT | O_APPEND | O_CLOEXEC, 0644);
+        if (fd >= 0) g_abort_fd = fd;
+    }
     void* warm[2];
     (void)backtrace(warm, 2);  // loads the unwinder now, not inside the handler
     struct sigaction sa;
@@ -75,6 +111,70 @@ void install_abort_backtrace() {
     sigemptyset(&sa.sa_mask);
     sa.sa_flags = SA_SIGINFO | SA_NODEFER;
     sigaction(SIGABRT, &sa, &g_previous_abort_action);
+    g_previous_terminate = std::set_terminate(&terminate_with_message);
+}
+
+// The engine shut down from its own worker thread.
+//  "task_owns_engine": a task holds the last reference to the engine it runs on; two more
+//      tasks are queued behind it.  Returns the order in which the three ran.
+//  "callback_drops_owner": an owner of an engine (as a process group is) is kept alive only
+//      by a Future callback; the engine's task completes the Work, the callback runs on the
+//      engine thread and is destroyed there, and with it the owner and its engine.
+std::vector<int> progress_self_shutdown(const std::string& mode) {
+    auto order = std::make_shared<std::vector<int>>();
+    auto mu = std::make_shared<std::mutex>();
+    auto push = [order, mu](int v) {
+        std::lock_guard<std::mutex> lk(*mu);
+        order->push_back(v);
+    };
+    auto settled = [&](size_t want) {
+        for (int i = 0; i < 500; ++i) {
+            {
+                std::lock_guard<std::mutex> lk(*mu);
+                if (order->size() >= want) break;
+            }
+            std::this_thread::sleep_for(std::chrono::milliseconds(10));
+        }
+        std::this_thread::sleep_for(std::chrono::milliseconds(30));  // lets the worker leave its loop
+        std::lock_guard<std::mutex> lk(*mu);
+        return *order;
+    };
+    if (mode == "task_owns_engine") {
+        auto engine = std::make_shared<mccl::Progress>();
+        engine->submit([engine, push] {
+            std::this_thread::sleep_for(std::chrono::milliseconds(40));  // until the caller has let go
+            push(1);
+        });
+        engine->submit([push] { push(2); });
+        engine->submit([push] { push(3); });
+        engine.reset();
+        return settled(3);
+    }
+    if (mode == "callback_drops_owner") {
+        struct Owner {
+            std::unique_ptr<mccl::Progress> engine = std::make_unique<mccl::Progress>();
+            std::function<void(int)> push;
+            ~Owner() {
+                engine->shutdown();
+                push(9);  // the owner's members are still whole here
+            }
+        };
+        auto owner = std::make_shared<Owner>();
+        owner->push = push;
+        auto work = c10::make_intrusive<mccl::WorkMCCL>(c10d::OpType::ALLREDUCE, std::vector<at::Tensor>{}, "mccl:test");
+        work->getFuture()->addCallback([owner, push](c10::ivalue::Future&) { push(1); });
+        mccl::Progress* engine = owner->engine.get();
+        engine->submit([work, push] {
+            std::this_thread::sleep_for(std::chrono::milliseconds(40));
+            work->finish();  // runs the callback here; the Future then drops it, and the owner with it
+            push(2);
+        });
+        engine->submit([push] { push(3); });
+        owner.reset();
+        work.reset();
+        return settled(4);
+    }
+    throw mccl::MCCLError("unknown mode " + mode);
 }
 
 // Submits n tasks; task i throws when bit i of throw_mask is set (i < 64).
@@ -366,6 +466,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         return mccl::log::enabled(level);
     });
     m.def("_test_progress_shutdown_while_task_needs_gil", &progress_shutdown_while_task_needs_gil);
+    m.def("_test_progress_self_shutdown", &progress_self_shutdown, py::arg("mode"),
+          py::call_guard<py::gil_scoped_release>());
+    m.def("_test_terminate", [](const std::string& what) {
+        // ends the process (tests run it in a child): an exception nobody catches, on a native thread
+        std::thread t([what] { throw mccl::MCCLError(what); });
+        t.join();
+    }, py::call_guard<py::gil_scoped_release>());
     m.def("_test_progress_submit_latency_us", &progress_submit_latency_us,
           py::call_guard<py::gil_scoped_release>());
     m.def("_test_work", &work_probe, py::arg("mode"), py::arg("wait_ms") = 1000,

@@ -5,10 +5,27 @@ import pytest
 
 # libmcclx checks every launch's pointers against their allocations when this is set
 os.environ.setdefault("MCCLX_VALIDATE", "1")
-# should the process ever abort, the extension prints the native stack of the thread that did it
-os.environ.setdefault("MCCL_ABORT_BACKTRACE", "1")
-
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _abort_log() -> str:
+    """Should the process ever abort, the extension writes the native stack of the thread that
+    did it, and the message of an uncaught C++ exception, to this file: file descriptor 2 is
+    pytest's capture file while a test runs, and what is written there dies with the process."""
+    for d in (os.path.join(ROOT, "gpurun_out"), os.environ.get("TMPDIR") or "/tmp"):
+        try:
+            os.makedirs(d, exist_ok=True)
+            path = os.path.join(d, "mccl_abort_backtrace.txt")
+            with open(path, "a"):
+                pass
+            return path
+        except OSError:
+            continue
+    return "1"
+
+
+os.environ.setdefault("MCCL_ABORT_BACKTRACE", _abort_log())
+
 for p in (ROOT, os.path.join(ROOT, "tests")):
     if p not in sys.path:
         sys.path.insert(0, p)

@@ -46,6 +46,42 @@ def test_same_observable_order_as_the_reference_engine(CX):
         assert CX._test_progress_order(n, mask, False) == list(buf[:k])
 
 
+# ---- the engine shut down from its own worker thread ---------------------------------------
+# (the reference leaves this open; a join of the calling thread throws inside a destructor and
+# std::terminate ends the process with SIGABRT on a native thread)
+
+def test_a_task_may_hold_the_last_reference_to_its_own_engine(CX):
+    """The engine is destroyed on its own worker, by the task that owned it: the tasks queued
+    behind that one still run, in order, and nothing aborts."""
+    assert CX._test_progress_self_shutdown("task_owns_engine") == [1, 2, 3]
+
+
+def test_a_future_callback_may_drop_the_owner_of_the_engine_it_runs_on(CX):
+    """An owner of an engine (as a process group is) dies on that engine's thread, when the
+    Future of a Work completed there drops the callback that kept it alive: the callback runs
+    (1), the owner's destructor shuts the engine down from its own thread, which runs the
+    queued task there and then (3) while the owner's members are still whole (9), and the
+    task that completed the Work goes on to its end (2)."""
+    assert CX._test_progress_self_shutdown("callback_drops_owner") == [1, 3, 9, 2]
+
+
+def test_an_uncaught_exception_on_a_native_thread_is_named_in_the_abort_file(tmp_path):
+    """std::terminate on a worker thread: the message and the native stack go to the file
+    MCCL_ABORT_BACKTRACE names (file descriptor 2 may belong to a test runner's capture)."""
+    import subprocess
+    import sys
+    log = tmp_path / "abort.txt"
+    env = dict(os.environ, MCCL_ABORT_BACKTRACE=str(log))
+    r = subprocess.run([sys.executable, "-c",
+                        "from mccl_amd import _C; _C._test_terminate('engine thread blew up')"],
+                       env=env, capture_output=True, text=True, timeout=120,
+                       cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert r.returncode == -6, (r.returncode, r.stderr[-500:])
+    text = log.read_text()
+    assert "std::terminate called with an uncaught exception: [MCCL] engine thread blew up" in text
+    assert "SIGABRT: native stack of the aborting thread" in text
+
+
 # ---- WorkMCCL: csrc/backend/WorkMCCL.cpp:46-104 --------------------------------
 
 def test_work_completion_states(CX):
