@@ -32,6 +32,15 @@
 
 namespace mccl {
 
+// Event-based completion: how far one rank's stream has already been put behind each of
+// the mesh's reduce queues (the id of the newest launch an event it waits for covers).
+struct WaitMarks {
+    std::mutex mu;
+    void* stream[2] = {nullptr, nullptr};
+    bool valid[2] = {false, false};
+    uint64_t upto[2] = {0, 0};
+};
+
 // What one rank contributes to a collective: raw device addresses plus the
 // parameters all ranks must agree on.
 struct Contribution {
@@ -48,6 +57,7 @@ struct Contribution {
     void* stream = nullptr;        // the rank's producer/consumer HIP stream
     void* work = nullptr;          // the rank's completion object, when the leader (or a later
                                    // launch) settles it instead of the rank itself
+    std::shared_ptr<WaitMarks> marks;  // the rank's record of what its stream already waits for
     int async = 0;                 // allreduce: event-based completion asked for (ranks must agree)
     int direct = 1;                // allreduce: read peers' fp32 tensors in place (rank 0's setting is used)
     int transport = 0;             // allreduce: 0 = peers read in place, 1 = pinned host wire, 2 = staged host wire

@@ -16,6 +16,7 @@
 #include "backend/HostWire.hpp"
 #include "backend/LocalMesh.hpp"
 #include "backend/Logging.hpp"
+#include "backend/Phases.hpp"
 #include "backend/Progress.hpp"
 #include "backend/WorkMCCL.hpp"
 
@@ -147,6 +148,7 @@ struct ProcessGroupMCCL::Shared : std::enable_shared_from_this<ProcessGroupMCCL:
         at::Tensor workspace;                  // wire copies / recv scratch of this call
         std::vector<c10::intrusive_ptr<WorkMCCL>> works;  // one per rank
         std::atomic<bool> launched{false};
+        std::atomic<uint64_t> flight{0};       // id of the launch that carries it (ids grow with every launch of the mesh)
         int queue = 0;
         uint64_t arrival = 0;
         std::vector<Span> spans;               // every byte range the launch reads or writes
@@ -164,6 +166,7 @@ struct ProcessGroupMCCL::Shared : std::enable_shared_from_this<ProcessGroupMCCL:
                                                  // blocked in a wait on the newest event, and a query from
                                                  // another thread would block with it)
     uint64_t arrivals = 0, next_flight = 1;
+    uint64_t newest_flight[2] = {0, 0};          // the last launch enqueued on each queue
     bool main_touched = true;                    // the main queue got work the second queue has not waited for
     std::vector<at::Tensor> workspace_pool;      // workspaces of finished buckets, for reuse
     std::unique_ptr<Progress> completer;
@@ -200,6 +203,10 @@ struct ProcessGroupMCCL::Shared : std::enable_shared_from_this<ProcessGroupMCCL:
         return *q ? alt : ctx;
     }
     mcclx_ctx* queue(int q) const { return q ? alt : ctx; }
+    uint64_t newest_on(int q) {
+        std::lock_guard<std::mutex> lk(amu);
+        return newest_flight[q];
+    }
 
     // A workspace for one asynchronous call (several may be in flight, each keeps its
     // own until it has finished).  One that comes back from a finished bucket has no
@@ -267,23 +274,32 @@ struct ProcessGroupMCCL::Shared : std::enable_shared_from_this<ProcessGroupMCCL:
             // itself should not time its stores (mcclx_set_hold; measured beside a stream of
             // copies: 27.7 us with the hold form, 24.1 us without)
             check_rc(mcclx_set_hold(queue(q), 0));
-            check_rc(mcclx_allreduce_replay_many(queue(q), all.data(), static_cast<uint32_t>(all.size())));
+            {
+                phases::Span ph(phases::kLaunch);
+                check_rc(mcclx_allreduce_replay_many(queue(q), all.data(), static_cast<uint32_t>(all.size())));
+            }
+            phases::Span ph(phases::kSubmit);
             check_rc(mcclx_event_record(queue(q), &ticket));
         } catch (...) {
             err = std::current_exception();
         }
+        const uint64_t id = next_flight++;
+        if (!err) newest_flight[q] = id;
         // only now: a rank that waits on one of these Works and finds it not launched takes
         // `amu` (flush_parked) and so gets behind this launch before it orders its stream
-        for (auto& b : buckets) b->launched = true;
+        for (auto& b : buckets) {
+            b->flight = id;
+            b->launched = true;
+        }
         if (err) {
             for (auto& b : buckets)
                 for (auto& w : b->works) w->finishWithException(err);
             std::rethrow_exception(err);
         }
-        const uint64_t id = next_flight++;
         flights[q].push_back(Flight{id, std::move(spans)});
         ++async_launches;
         async_buckets += buckets.size();
+        phases::Span ph_submit(phases::kSubmit);
         if (!completer) completer = std::make_unique<Progress>();
         mcclx_ctx* c = queue(q);
         // The task keeps this object alive while it runs: settling a Work runs the callbacks of
@@ -295,11 +311,15 @@ struct ProcessGroupMCCL::Shared : std::enable_shared_from_this<ProcessGroupMCCL:
         std::shared_ptr<Shared> self = weak_from_this().lock();
         completer->submit([this, self, c, q, id, ticket, buckets = std::move(buckets)]() mutable {
             std::exception_ptr failure;
-            try {
-                check_rc(mcclx_event_wait(c, ticket));
-            } catch (...) {
-                failure = std::current_exception();
+            {
+                phases::Span ph(phases::kCompleterWait);
+                try {
+                    check_rc(mcclx_event_wait(c, ticket));
+                } catch (...) {
+                    failure = std::current_exception();
+                }
             }
+            phases::Span ph_settle(phases::kSettle);
             {
                 std::lock_guard<std::mutex> lk(amu);
                 for (auto it = flights[q].begin(); it != flights[q].end(); ++it)
@@ -504,6 +524,7 @@ ProcessGroupMCCL::ProcessGroupMCCL(c10::intrusive_ptr<c10d::Store> store, int ra
         MCCL_CHECK(shared_ != nullptr, "mesh context already destroyed");
     }
     ctx_ = shared_->ctx;
+    wait_marks_ = std::make_shared<WaitMarks>();
     engine_ = std::make_unique<Progress>();
     MCCL_INFO("rank %d of %d joined in-process mesh %s on GPU %d (%d CUs)", rank, size, mesh_key_.c_str(), device_,
               mcclx_device_cus(ctx_));
@@ -667,6 +688,7 @@ int env_transport() {
 c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tensor>& tensors,
                                                            const c10d::AllreduceOptions& opts) {
     if (getSize() == 1) return make_completed(c10d::OpType::ALLREDUCE, tensors, "mccl:allreduce");
+    phases::Span ph_build(phases::kBuild);
     const int world = getSize();
     int transport = 0;
     bool async = false;
@@ -678,7 +700,10 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
         knob_error = e.what();
     }
     c10::intrusive_ptr<WorkMCCL> work;
-    if (async) work = c10::make_intrusive<WorkMCCL>(c10d::OpType::ALLREDUCE, tensors, "mccl:allreduce");
+    if (async) {
+        phases::Span ph(phases::kWorkMake);
+        work = c10::make_intrusive<WorkMCCL>(c10d::OpType::ALLREDUCE, tensors, "mccl:allreduce");
+    }
 
     // A rank whose own checks fail still goes to the meeting point, carrying the
     // message, so that the whole group fails at once instead of waiting for it.
@@ -717,6 +742,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
     c.direct = env_direct() ? 1 : 0;
     c.transport = transport;
     c.work = work.get();
+    c.marks = wait_marks_;
     flush_engine_();
 
     if (transport != 0) {
@@ -749,7 +775,15 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
 
     auto shared = shared_;
     const int device = device_;
+    ph_build.stop();
+    phases::Span ph_meet(phases::kMeet);
     meet(std::move(c), [shared, world, device](const std::vector<Contribution>& all) {
+        const auto leader_t0 = std::chrono::steady_clock::now();
+        struct OffMeet {  // what the last arrival does here is not time spent meeting
+            std::chrono::steady_clock::time_point t0;
+            ~OffMeet() { phases::discount(phases::kMeet, std::chrono::steady_clock::now() - t0); }
+        } off_meet{leader_t0};
+        phases::Span ph_checks(phases::kLeaderChecks);
         const size_t nt = all[0].dst.size();
         const bool async = all[0].async != 0;
         int qsel = 0;
@@ -767,11 +801,16 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
         // mps_stream_sync, :172 -- once per distinct stream: ranks on one stream (threads
         // that all use torch's default stream) are covered by one wait, and a wait costs
         // the host about ten microseconds
-        for (int r = 0; r < world; ++r) {
-            bool seen = false;
-            for (int q = 0; q < r; ++q) seen = seen || all[q].stream == all[r].stream;
-            if (!seen) check_rc(mcclx_queue_wait_stream(ctx, all[r].stream));
+        {
+            ph_checks.stop();
+            phases::Span ph(phases::kStreamWait);
+            for (int r = 0; r < world; ++r) {
+                bool seen = false;
+                for (int q = 0; q < r; ++q) seen = seen || all[q].stream == all[r].stream;
+                if (!seen) check_rc(mcclx_queue_wait_stream(ctx, all[r].stream));
+            }
         }
+        phases::Span ph_checks2(phases::kLeaderChecks);
         // one replay per tensor of the list; the reference runs them one after another
         // (ProcessGroupMCCL.cpp:122-168), here a list is issued together so that
         // entries sharing a plan need one launch per phase for all of them
@@ -845,27 +884,56 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
             // released on the completer thread, which must never be the one to tear the group down)
             std::weak_ptr<Shared::Bucket> weak = bucket;
             std::weak_ptr<Shared> weak_shared = shared;
-            for (auto& w : bucket->works)
-                w->setWaitHook([weak_shared, weak, device] {
+            for (int r = 0; r < world; ++r) {
+                // A stream that was put behind a launch of a queue is behind every earlier launch
+                // of that queue as well: a rank that waits for its buckets one after another pays
+                // for one event per queue, not one per bucket (an event record plus a wait of
+                // torch's legacy stream cost the host 20-35 us).
+                std::shared_ptr<WaitMarks> marks = all[r].marks;
+                bucket->works[static_cast<size_t>(r)]->setWaitHook([weak_shared, weak, device, marks] {
+                    phases::Span ph(phases::kWaitHook);
                     auto sh = weak_shared.lock();
                     if (!sh) return;  // the group is gone: its destructor has drained the queue
                     auto b = weak.lock();
                     if (!b) return;   // settled and released: nothing left to order against
                     if (!b->launched) sh->flush_parked(b->queue);
-                    check_rc(mcclx_stream_wait_queue(sh->queue(b->queue), dev::current_stream(device)));
+                    const int q = b->queue;
+                    const uint64_t id = b->flight.load();
+                    void* stream = dev::current_stream(device);
+                    if (marks) {
+                        std::lock_guard<std::mutex> lk(marks->mu);
+                        if (id != 0 && marks->stream[q] == stream && marks->valid[q] && marks->upto[q] >= id) return;
+                    }
+                    const uint64_t newest = sh->newest_on(q);  // enqueued before the event below is
+                    check_rc(mcclx_stream_wait_queue(sh->queue(q), stream));
+                    if (marks) {
+                        std::lock_guard<std::mutex> lk(marks->mu);
+                        marks->stream[q] = stream;
+                        marks->valid[q] = true;
+                        marks->upto[q] = std::max(newest, id);
+                    }
                 });
+            }
+            ph_checks2.stop();
             shared->submit_bucket(bucket);
             return;
         }
+        ph_checks2.stop();
         // The reference's allreduce is synchronous (ProcessGroupMCCL.cpp:170-185): when
         // it returns, every rank's tensor holds the result and the queue is drained.
-        if (nt == 1)
-            shared->allreduce(reps[0]);  // a single bucket: recorded and replayed when it comes again
-        else
-            check_rc(mcclx_allreduce_replay_many(ctx, reps.data(), static_cast<uint32_t>(nt)));
+        {
+            phases::Span ph(phases::kLaunch);
+            if (nt == 1)
+                shared->allreduce(reps[0]);  // a single bucket: recorded and replayed when it comes again
+            else
+                check_rc(mcclx_allreduce_replay_many(ctx, reps.data(), static_cast<uint32_t>(nt)));
+        }
+        phases::Span ph(phases::kDrain);
         check_rc(mcclx_queue_drain(ctx));  // mccl_queue_drain, :178
     });
+    ph_meet.stop();
     if (async) return work;
+    phases::Span ph_work(phases::kWorkMake);
     return make_completed(c10d::OpType::ALLREDUCE, tensors, "mccl:allreduce");
 }
 

@@ -32,6 +32,7 @@ class Progress;
 class LocalMesh;
 class HostWire;
 struct Contribution;
+struct WaitMarks;
 
 class ProcessGroupMCCL : public c10d::Backend {
     using Tensors = std::vector<at::Tensor>;
@@ -96,6 +97,7 @@ private:
     std::shared_ptr<LocalMesh> mesh_;
     std::string mesh_key_;
     std::unique_ptr<Progress> engine_;
+    std::shared_ptr<WaitMarks> wait_marks_;  // event-based allreduce: what this rank's stream already waits for
     std::unique_ptr<HostWire> host_wire_;  // MCCL_WIRE=host|staged: this rank's end of the byte transport
     int last_algo_ = -1;
 };

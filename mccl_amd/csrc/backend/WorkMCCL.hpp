@@ -15,6 +15,7 @@
 
 #include <ATen/ATen.h>
 
+#include <atomic>
 #include <chrono>
 #include <condition_variable>
 #include <exception>
@@ -65,6 +66,7 @@ private:
     mutable std::mutex mu_;
     std::condition_variable settled_cv_;
     State state_ = State::Pending;
+    std::atomic<bool> done_{false};  // state_ != Pending, readable without the lock (polled by wait())
     std::exception_ptr error_;
 };
 

@@ -32,6 +32,7 @@
 #include "backend/Errors.hpp"
 #include "backend/LocalMesh.hpp"
 #include "backend/Logging.hpp"
+#include "backend/Phases.hpp"
 #include "backend/ProcessGroupMCCL.hpp"
 #include "backend/Progress.hpp"
 #include "backend/WorkMCCL.hpp"
@@ -459,6 +460,15 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         return p ? p->launchCount() : uint64_t(0);
     });
 
+    m.def("_phase_stats", [](bool reset) {
+        // phase -> (calls, total microseconds) since the last reset; all zero unless MCCL_PHASE_STATS=1
+        py::dict d;
+        for (int p = 0; p < mccl::phases::kCount; ++p)
+            d[mccl::phases::name(p)] = py::make_tuple(mccl::phases::totals().calls[p].load(),
+                                                      static_cast<double>(static_cast<int64_t>(mccl::phases::totals().ns[p].load())) * 1e-3);
+        if (reset) mccl::phases::reset();
+        return d;
+    }, py::arg("reset") = false);
     m.def("_test_progress_order", &progress_order, py::arg("n"), py::arg("throw_mask") = 0,
           py::arg("use_destructor") = false, py::call_guard<py::gil_scoped_release>());
     m.def("_test_log", [](int level, const std::string& text) {
