@@ -515,6 +515,24 @@ def backend_extras(torch, W):
             # the same with the ranks as native threads: what the interpreter lock shared by
             # three Python rank threads adds to the figure above
             out[f"c2_backend_{mode}_native_ranks_us_per_bucket"] = round(max(CX._allreduce_rate(3, numel, nb, 4)), 1)
+        # small buckets, event-based, native rank threads: 16 buckets of 1 MiB back to back, with the
+        # default gathering of small buckets into one launch and without it
+        os.environ["MCCL_ALLREDUCE_ASYNC"] = "1"
+        saved_cb = os.environ.get("MCCL_COALESCE_BELOW")
+        try:
+            small = {}
+            for name, below in (("gathered", None), ("one_launch_each", "0")):
+                if below is None:
+                    os.environ.pop("MCCL_COALESCE_BELOW", None)
+                else:
+                    os.environ["MCCL_COALESCE_BELOW"] = below
+                small[name] = round(max(CX._allreduce_rate(3, (1 << 20) // 4, 16, 6)), 1)
+            out["backend_async_native_ranks_16_buckets_of_1MiB_us_per_bucket"] = small
+        finally:
+            if saved_cb is None:
+                os.environ.pop("MCCL_COALESCE_BELOW", None)
+            else:
+                os.environ["MCCL_COALESCE_BELOW"] = saved_cb
         os.environ.pop("MCCL_ALLREDUCE_ASYNC", None)
 
         os.environ.update({"MCCL_ALLREDUCE_ALGO": "ring", "MCCL_WIRE": "host"})
@@ -703,6 +721,20 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
         reps = max(10, min(200, (16 << 30) // (n * 12)))
         ms, _ = measure(sz_step, reps, 5)
         sweep[f"{mib}MiB"] = {"us": round(ms / reps * 1e3, 2), "GBps": round(gbs(n * 12, ms / reps), 1)}
+        if mib == 1:
+            # four 1 MiB buckets in ONE launch (12 segments by value): what the event-based path
+            # issues for small buckets that gather while a launch is in flight
+            def four(i, bufs=bufs, ch=ch, ncopies=ncopies):
+                segs = []
+                for b in range(4):
+                    ts, ws = bufs[(4 * i + b) % ncopies]
+                    segs += [K.make_seg(ts[R].data_ptr() + 4 * st, 0,
+                                        [ts[R].data_ptr() + 4 * st] + [ws[p].data_ptr() + 2 * st for p in range(world) if p != R], c)
+                             for R, (st, c, _, _) in enumerate(ch)]
+                q.fold(plan, segs)
+            ms, _ = measure(four, reps, 5)
+            sweep["4x1MiB_in_one_launch"] = {"us": round(ms / reps * 1e3, 2), "us_per_bucket": round(ms / reps * 1e3 / 4, 2),
+                                             "GBps": round(gbs(4 * n * 12, ms / reps), 1)}
         del bufs
     out["fold_by_bucket_size"] = sweep
 

@@ -150,6 +150,7 @@ struct ProcessGroupMCCL::Shared : std::enable_shared_from_this<ProcessGroupMCCL:
         std::atomic<bool> launched{false};
         std::atomic<uint64_t> flight{0};       // id of the launch that carries it (ids grow with every launch of the mesh)
         int queue = 0;
+        bool small = false;                    // below MCCL_COALESCE_BELOW: see submit_bucket
         uint64_t arrival = 0;
         std::vector<Span> spans;               // every byte range the launch reads or writes
     };
@@ -178,6 +179,7 @@ struct ProcessGroupMCCL::Shared : std::enable_shared_from_this<ProcessGroupMCCL:
         if (const char* m = std::getenv("MCCL_GRAPH_MIN_LAUNCHES")) graph_min_launches = std::strtoull(m, nullptr, 10);
         const char* q = std::getenv("MCCL_ASYNC_QUEUES");
         if (q && q[0] == '1') queues = 1;
+        if (const char* c = std::getenv("MCCL_COALESCE_BELOW")) coalesce_below = std::strtoull(c, nullptr, 10);
     }
     ~Shared() {
         try {
@@ -195,10 +197,20 @@ struct ProcessGroupMCCL::Shared : std::enable_shared_from_this<ProcessGroupMCCL:
 
     static constexpr size_t kDepth = 2;  // launches in flight per queue: the next one is behind the one that runs
 
+    // Small buckets.  A launch of a 1 MiB bucket keeps the device busy for under 3 us (15 % of
+    // what the memory system can do: a launch's fixed cost dominates), four of them in one
+    // launch for 4 us.  A bucket of fewer bytes than this (per rank; MCCL_COALESCE_BELOW,
+    // default 8 MiB, 0 = off) therefore goes out at once only when its queue is empty; while
+    // ANY launch of that queue is still in flight it is parked, and everything parked goes out
+    // as one launch when that one has finished (or a rank waits for one of them) -- the window
+    // in which buckets gather is the time the completer needs to see a launch end, some 20 us.
+    // Small buckets all take the main queue: two queues would halve what gathers on either.
+    uint64_t coalesce_below = 8ull << 20;
+
     // Which queue the next event-based allreduce goes to, and that queue.
-    mcclx_ctx* pick_queue(int* q) {
+    mcclx_ctx* pick_queue(int* q, bool small) {
         std::lock_guard<std::mutex> lk(amu);
-        *q = queues == 2 ? static_cast<int>(arrivals & 1) : 0;
+        *q = (queues == 2 && !small) ? static_cast<int>(arrivals & 1) : 0;
         if (*q == 1 && !alt) check_rc(mcclx_init(device, &alt));
         return *q ? alt : ctx;
     }
@@ -355,7 +367,7 @@ struct ProcessGroupMCCL::Shared : std::enable_shared_from_this<ProcessGroupMCCL:
         b->arrival = arrivals++;
         const int q = b->queue;
         // (a launch that finishes after this check takes `amu` after us and finds the bucket parked)
-        if (parked[q].empty() && flights[q].size() < kDepth) {
+        if (parked[q].empty() && flights[q].size() < (b->small ? size_t(1) : kDepth)) {
             launch_locked(q, {std::move(b)});
             return;
         }
@@ -788,10 +800,16 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
         const bool async = all[0].async != 0;
         int qsel = 0;
         mcclx_ctx* ctx = shared->ctx;
-        if (async)
-            ctx = shared->pick_queue(&qsel);
-        else
+        bool small = false;
+        if (async) {
+            uint64_t bytes = 0;
+            for (size_t i = 0; i < nt && i < all[0].numel.size() && i < all[0].dtype.size(); ++i)
+                bytes += all[0].numel[i] * (all[0].dtype[i] == MCCLX_F32 ? 4u : 2u);
+            small = bytes < shared->coalesce_below;
+            ctx = shared->pick_queue(&qsel, small);
+        } else {
             shared->begin_main_work();
+        }
         for (int r = 0; r < world; ++r) {
             MCCL_CHECK(all[r].dst.size() == nt, "allreduce: ranks passed different numbers of tensors");
             MCCL_CHECK(all[r].op == all[0].op && all[r].wire_bf16 == all[0].wire_bf16,
@@ -862,6 +880,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupMCCL::allreduce(std::vector<at::Tenso
         }
         if (async) {
             bucket->queue = qsel;
+            bucket->small = small;
             for (size_t i = 0; i < nt; ++i) {
                 const uint64_t tb = reps[i].numel * (reps[i].dtype == MCCLX_F32 ? 4u : 2u);
                 for (int r = 0; r < world; ++r) {

@@ -352,6 +352,7 @@ def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypat
     monkeypatch.setenv("MCCL_ASYNC_QUEUES", str(queues))
     monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "butterfly")
     monkeypatch.setenv("MCCL_WIRE_DTYPE", "bf16")
+    monkeypatch.setenv("MCCL_COALESCE_BELOW", "0")   # the queue mechanics alone (small buckets gather: see the next test)
     world = 3
     sizes = [6_553_600, 1_000_003, 70_001, 1_000_003, 33, 4097, 250_000]
     rng = np.random.default_rng(31)
@@ -402,6 +403,56 @@ def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypat
     assert k1 - k0 == (1 if direct else 2) * (l1 - l0), \
         "a launch of several buckets is one fold that also hands out the result (behind one encode without MCCL_DIRECT), once"
     assert all(all(out[r][2]) for r in range(world)), "a Work was complete when allreduce returned"
+
+
+@pytest.mark.parametrize("below,launches", [(None, 2), ("0", None)])
+def test_small_event_based_buckets_gather_behind_a_launch_in_flight(CX, U, monkeypatch, below, launches):
+    """Buckets under MCCL_COALESCE_BELOW (8 MiB by default) take the main queue and are parked
+    while ANY launch of it is in flight; what has gathered goes out as one launch.  Eight 1 MiB
+    buckets issued behind a busy stream: the first goes out at once, the other seven together --
+    two launches, against at least three with the gathering off (two launches in flight on each
+    of two queues, the rest behind them).  Results are the oracle's, bit for bit, either way."""
+    monkeypatch.setenv("MCCL_ALLREDUCE_ASYNC", "1")
+    monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "butterfly")
+    monkeypatch.setenv("MCCL_WIRE_DTYPE", "bf16")
+    if below is None:
+        monkeypatch.delenv("MCCL_COALESCE_BELOW", raising=False)
+    else:
+        monkeypatch.setenv("MCCL_COALESCE_BELOW", below)
+    world, nb, n = 3, 8, (1 << 20) // 4
+    rng = np.random.default_rng(77)
+    xs = [[(rng.standard_normal(n + 3 * i) * 1e-3).astype(np.float32) for _ in range(world)] for i in range(nb)]
+
+    def fn(r, pg):
+        ts = [U.to_dev(x[r], F32) for x in xs]
+        big = torch.empty(1 << 30, dtype=torch.uint8, device="cuda") if r == 0 else None
+        torch.cuda.current_stream().synchronize()
+        before = CX._async_stats(pg)
+        if r == 0:
+            for _ in range(100):   # some 25 ms of copies: the first launch waits for this stream on the device
+                big[: 1 << 29].copy_(big[1 << 29:])
+        o = dist.AllreduceOptions(); o.reduceOp = dist.ReduceOp.AVG
+        works = [pg.allreduce([t], o) for t in ts]
+        for w in works:
+            assert w.wait(datetime.timedelta(seconds=60))   # with a timeout: blocks the host until settled
+            assert w.is_completed() and w.is_success()
+        torch.cuda.current_stream().synchronize()
+        return ts, before, CX._async_stats(pg)
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for i in range(nb):
+        want = [x.copy() for x in xs[i]]
+        rc, used = orc.pg_allreduce(want, F32, AVG, wire_bf16=True, env_algo="butterfly", threads=orc.max_threads())
+        assert rc == 0 and used == BUTTERFLY
+        for r in range(world):
+            U.assert_same_bits(out[r][0][i], want[r], F32, f"bucket {i} rank {r}")
+    (l0, b0), (l1, b1) = out[0][1], out[0][2]
+    assert b1 - b0 == nb
+    if launches is not None:
+        assert l1 - l0 == launches, "the seven buckets behind the first went out together"
+    else:
+        assert 3 <= l1 - l0 <= nb
 
 
 @pytest.mark.parametrize("queues", [1, 2])

@@ -522,3 +522,12 @@ def test_fan_out_validation(K):
     with pytest.raises(Exception) as e:                                 # fan-out without `out`
         q.fold(K.make_plan(BF16, 2, fanout=1), [K.make_seg(0, t.data_ptr(), [t.data_ptr()] * 3, 16)])
     assert "fan-out needs `out`" in str(e.value)
+    # a destination may BE an operand; one that overlaps an operand at another offset would be
+    # read by some lanes after others have written it (checked under MCCLX_VALIDATE, which the tests set)
+    a, b = torch.zeros(64, device="cuda"), torch.zeros(64, device="cuda")
+    q.fold(K.make_plan(F32, 2, fanout=1), [K.make_seg(a.data_ptr(), 0, [a.data_ptr(), b.data_ptr(), b.data_ptr()], 16)])
+    with pytest.raises(Exception) as e:
+        q.fold(K.make_plan(F32, 2, fanout=1),
+               [K.make_seg(a.data_ptr(), 0, [a.data_ptr(), b.data_ptr(), b.data_ptr() + 8], 16)])
+    assert "overlaps operand in[1]" in str(e.value)
+    K.hip_sync()

@@ -235,3 +235,23 @@ def test_results_do_not_depend_on_the_gate(env, queues, knobs):
         check_outputs(U, checks, f"gate knobs {knobs}")
     finally:
         q.close()
+
+
+def test_the_gate_follows_the_device_and_the_knobs_override_it(monkeypatch):
+    """The rate behind the hold form's gate is measured when the first context of the process
+    is made (two read-only launches over scratch memory): on MI355X it lands near 70,000 bytes
+    per 10 ns tick.  MCCLX_HOLD_BYTES_PER_TICK overrides it for contexts made afterwards, and
+    MCCLX_HOLD_CALIBRATE=0 cannot undo a measurement already cached for the device."""
+    from mccl_amd import kernels as K
+    q = K.ReduceQueue(0)
+    lat, bpt, measured = q.hold_model()
+    q.close()
+    assert measured and lat == 40 and 50_000 <= bpt <= 95_000, (lat, bpt, measured)
+    monkeypatch.setenv("MCCLX_HOLD_BYTES_PER_TICK", "65432")
+    q = K.ReduceQueue(0)
+    assert q.hold_model() == (40, 65432, False)
+    q.close()
+    monkeypatch.delenv("MCCLX_HOLD_BYTES_PER_TICK")
+    q = K.ReduceQueue(0)
+    assert q.hold_model() == (lat, bpt, True), "one measurement per device and process"
+    q.close()

@@ -107,3 +107,68 @@ def test_noalloc_limit_and_launch_only(env):
     K.hip_sync()
     assert torch.cuda.mem_get_info()[0] == free_before
     assert torch.equal(out, a + 1)
+
+
+def test_noalloc_ragged_launch_of_few_segments_takes_the_static_table(env):
+    """Up to 32 segments travel in the kernel arguments only when they are of similar length:
+    one long segment among many short ones would launch (longest x segments) blocks, most of
+    them idle, so such a launch goes through the static table like mcclx_fold_batched's goes
+    through an uploaded one (same rule).  Seen from outside: more than one kernel launch."""
+    L, K, U = env
+    rng = np.random.default_rng(5)
+    q = K._q(None)
+    counts = np.array([900_000] + [300] * 19)
+    before = q.launch_count()
+    pairs, _ = _case(L, K, U, rng, 20, counts, orc.F32, 2, L.IO_PURE, None)
+    _same(pairs, "20 ragged segments")
+    # fold_batched: 1 launch (its table is uploaded by a copy); noalloc: writer launch(es) + the fold
+    assert q.launch_count() - before >= 3
+    before = q.launch_count()
+    pairs, _ = _case(L, K, U, rng, 20, np.full(20, 5000), orc.F32, 2, L.IO_PURE, None)
+    _same(pairs, "20 even segments")
+    assert q.launch_count() - before == 2, "even segments travel by value: one launch per entry point"
+
+
+def test_noalloc_concurrent_entry_from_two_contexts_is_refused_not_interleaved(env):
+    """Every context on a GPU shares the one static table.  A call that enters while another
+    thread's call is still writing descriptors is refused with MCCLX_ERR_STATE instead of
+    interleaving its writer launches with the other's.  Two threads, each with a context of its
+    own, hammer the entry point with the SAME segments (what overlaps on the device -- which
+    the host cannot see, and which the entry point leaves to its callers -- then writes the
+    same bytes): every call returns OK or ERR_STATE, and the result is right throughout."""
+    import threading
+    L, K, U = env
+    nseg, n, rounds = 40, 257, 150
+    plan = K.make_plan(orc.F32, 2)
+    a = torch.arange(nseg * n, dtype=torch.float32, device="cuda")
+    b = torch.full((nseg * n,), 2.0, device="cuda")
+    out = torch.zeros_like(a)
+    segs = [K.make_seg(out.data_ptr() + 4 * n * i, 0, [a.data_ptr() + 4 * n * i, b.data_ptr() + 4 * n * i], n)
+            for i in range(nseg)]
+    arr = (L.Seg * nseg)(*segs)
+    torch.cuda.synchronize()
+    errs, codes = [], [set(), set()]
+    start = threading.Barrier(2)
+
+    def worker(w):
+        try:
+            torch.cuda.set_device(0)
+            q = K.ReduceQueue(0)
+            start.wait()
+            for _ in range(rounds):
+                rc = L.lib().mcclx_fold_batched_noalloc(q.handle, C.byref(plan), arr, nseg)
+                codes[w].add(rc)
+                if rc == L.ERR_STATE:
+                    assert "static descriptor table" in L.last_error()
+            q.drain()
+            q.close()
+        except BaseException as e:  # noqa: BLE001
+            errs.append(e)
+
+    ts = [threading.Thread(target=worker, args=(w,)) for w in range(2)]
+    [t.start() for t in ts]
+    [t.join(300) for t in ts]
+    assert not errs, errs
+    assert codes[0] | codes[1] <= {L.OK, L.ERR_STATE} and L.OK in codes[0] and L.OK in codes[1]
+    torch.cuda.synchronize()
+    assert torch.equal(out, a + 2.0)
