@@ -5,6 +5,7 @@
 #endif
 
 #include <algorithm>
+#include <chrono>
 #include <cstring>
 
 #include "backend/Device.hpp"
@@ -162,7 +163,13 @@ void HostWire::allreduce(void* tensor, int dtype, uint64_t numel, int op, int al
         if (p.owner == me) mine = &p;
         max_count = std::max(max_count, p.count);
     }
-    stats_ = Stats{stats_.calls + 1, 0, 0, 0, 0.0, 0};
+    stats_ = Stats{stats_.calls + 1, 0, 0, 0, 0.0, 0, {0, 0, 0, 0, 0}};
+    auto leg_t0 = std::chrono::steady_clock::now();
+    auto leg_done = [&](int leg) {
+        const auto now = std::chrono::steady_clock::now();
+        stats_.leg_ms[leg] = std::chrono::duration<double, std::milli>(now - leg_t0).count();
+        leg_t0 = now;
+    };
 
     // buffers: what this rank sends (wire form, laid out like the tensor), what it
     // receives for its own chunk (one slot per peer), what it receives in the allgather leg
@@ -215,6 +222,7 @@ void HostWire::allreduce(void* tensor, int dtype, uint64_t numel, int op, int al
         if (!segs.empty()) check_rc(mcclx_fold_batched(ctx, &enc, segs.data(), static_cast<uint32_t>(segs.size())));
         check_rc(mcclx_queue_drain(ctx));  // the bytes are in host memory (Pinned) before the wire reads them
     }
+    leg_done(0);
 
     // ---- 2. reduce-scatter leg of the wire: my operand of every other chunk goes to its owner ...
     auto send_piece = [&](int to, const Piece& p) {
@@ -247,6 +255,7 @@ void HostWire::allreduce(void* tensor, int dtype, uint64_t numel, int op, int al
             recv_into(q, at(recv_a_dev, off), recv_a_host ? recv_a_host + off : nullptr, mine->count * es);
         }
 
+    leg_done(1);
     // ---- 3. one fold of all operands of my chunk, in the schedule's order
     if (mine) {
         mcclx_plan plan;
@@ -288,6 +297,7 @@ void HostWire::allreduce(void* tensor, int dtype, uint64_t numel, int op, int al
         check_rc(mcclx_queue_drain(ctx));  // every reduce complete before the next send reads it
     }
 
+    leg_done(2);
     // ---- 4. allgather leg: my reduced chunk goes to every peer, theirs arrive and are cast on arrival
     if (mine) {
         if (staged) {  // staged once, handed to every peer (the transport copies it)
@@ -332,8 +342,10 @@ void HostWire::allreduce(void* tensor, int dtype, uint64_t numel, int op, int al
             check_rc(mcclx_copy(ctx, at(tensor, p.start * ts), src, p.count * es));
         }
     }
+    leg_done(3);
     if (!dsegs.empty()) check_rc(mcclx_fold_batched(ctx, &dec, dsegs.data(), static_cast<uint32_t>(dsegs.size())));
     check_rc(mcclx_queue_drain(ctx));  // mccl_queue_drain, ProcessGroupMCCL.cpp:178
+    leg_done(4);
 }
 
 }  // namespace mccl

@@ -48,6 +48,9 @@ public:
         uint64_t fold_hbm_bytes = 0;       // bytes the fold read from and wrote to HBM
         double fold_ms = 0.0;
         uint64_t wire_bytes_sent = 0;      // bytes this rank handed to the transport in the last call
+        // host wall-clock milliseconds of the last call's legs: wire form of what is sent (encode,
+        // drained), reduce-scatter leg of the wire, fold (drained), allgather leg, casts on arrival
+        double leg_ms[5] = {0, 0, 0, 0, 0};
     };
 
     HostWire(std::shared_ptr<LocalMesh> mesh, int rank, int device, std::chrono::milliseconds timeout);

@@ -575,7 +575,8 @@ std::vector<double> ProcessGroupMCCL::wireStats() const {
     if (!host_wire_) return {};
     const HostWire::Stats& s = host_wire_->stats();
     return {static_cast<double>(s.calls), static_cast<double>(s.fold_elems), static_cast<double>(s.fold_peer_bytes),
-            static_cast<double>(s.fold_hbm_bytes), s.fold_ms, static_cast<double>(s.wire_bytes_sent)};
+            static_cast<double>(s.fold_hbm_bytes), s.fold_ms, static_cast<double>(s.wire_bytes_sent),
+            s.leg_ms[0], s.leg_ms[1], s.leg_ms[2], s.leg_ms[3], s.leg_ms[4]};
 }
 
 void* ProcessGroupMCCL::my_stream() const {

@@ -77,7 +77,8 @@ public:
     std::pair<uint64_t, uint64_t> asyncStats() const;
     uint64_t launchCount() const;
     // The last host-wire allreduce of this rank (MCCL_WIRE=host|staged): elements folded, bytes of
-    // peer operands the fold read, device milliseconds of the fold launch, bytes handed to the wire.
+    // peer operands the fold read, device milliseconds of the fold launch, bytes handed to the wire,
+    // then the host milliseconds of its five legs (wire form, reduce-scatter leg, fold, allgather leg, casts).
     std::vector<double> wireStats() const;
 
 private:

@@ -697,10 +697,18 @@ __global__ void __launch_bounds__(kHoldBlock) fold_few_hold_kernel(FewArgs a, ui
 #endif
 }
 
-// Plans with a reads-then-writes form: sums of two to four operands, rounding after every step.
+// Plans with a reads-then-writes form: sums of two to four operands, rounding after every step,
+// and the wire encode (one fp32 operand in, its bf16 form out: the first launch of every
+// schedule that sends bf16 copies; ten 16-byte packets per lane cover three 25 MiB tensors).
 template <class C>
-constexpr bool kHoldPlan = C::K >= 2 && C::K <= 4 && C::OP == MCCLX_SUM && C::ACC == MCCLX_ACC_STEP &&
-                           C::TOPO == MCCLX_TOPO_FOLD;
+constexpr bool kHoldEncode = C::K == 1 && C::IO == MCCLX_IO_OWN_FIRST_F32 && C::ACC == MCCLX_ACC_STEP;
+#ifndef MCCLX_HOLD_ENCODE_EARLY
+#define MCCLX_HOLD_ENCODE_EARLY 105
+#endif
+constexpr uint64_t kHoldEncodeEarlyPct = MCCLX_HOLD_ENCODE_EARLY;
+template <class C>
+constexpr bool kHoldPlan = ((C::K >= 2 && C::K <= 4) || kHoldEncode<C>) && C::OP == MCCLX_SUM &&
+                           C::ACC == MCCLX_ACC_STEP && C::TOPO == MCCLX_TOPO_FOLD;
 
 // Blocks of one generation: what the device holds at once of this kernel.
 template <class C, int T, int HB, bool FAN>
@@ -746,14 +754,24 @@ static bool try_hold(hipStream_t st, FewArgs& a, uint64_t maxc, const LaunchPara
     // measured break-even: 10 MiB read for a fold with one output, half as much again for one that
     // writes as much as it reads (fan-out)
     if (read_bytes < (FAN ? lp.hold_min_read_bytes * 3 / 2 : lp.hold_min_read_bytes)) return false;
+    // The encode: measured on 1-8 tensors of 1-40 MiB, the form wins 4-10 % from three tensors and
+    // 18 MiB read on (three of 25 MiB: 20.6 -> 19.0 us); on one or two tensors it ties or loses.
+    if constexpr (kHoldEncode<C>)
+        if (a.nseg < 3 || read_bytes < lp.hold_min_read_bytes * 9 / 5) return false;
     uint64_t ticks = lp.hold_latency_ticks + read_bytes / lp.hold_bytes_per_tick;
+    // the encode writes half of what it reads and does best with its stores a little early
+    if constexpr (kHoldEncode<C>) ticks = lp.hold_latency_ticks + read_bytes * 100 / (lp.hold_bytes_per_tick * kHoldEncodeEarlyPct);
     const uint32_t gate = ticks > 100000 ? 100000u : (uint32_t)ticks;  // a millisecond at most
     const uint64_t packets = (maxc + C::E - 1) / C::E;
     // A fold with one output takes four packets per lane if that covers it.  One that writes as
     // much as it reads (fan-out) does better with five and fewer waves: the one-launch allreduce
     // of a 25 MiB bucket 26.5 us against 27.6 us (of a 16 MiB bucket 17.4 against 17.2 us).
-    const bool took = FAN ? (hold_launch<C, 5, 512, FAN>(st, a, packets, gate, lp) || hold_launch<C, 4, 512, FAN>(st, a, packets, gate, lp))
-                          : (hold_launch<C, 4, 512, FAN>(st, a, packets, gate, lp) || hold_launch<C, 5, 512, FAN>(st, a, packets, gate, lp));
+    bool took;
+    if constexpr (kHoldEncode<C>)
+        took = hold_launch<C, 10, 512, false>(st, a, packets, gate, lp);
+    else
+        took = FAN ? (hold_launch<C, 5, 512, FAN>(st, a, packets, gate, lp) || hold_launch<C, 4, 512, FAN>(st, a, packets, gate, lp))
+                   : (hold_launch<C, 4, 512, FAN>(st, a, packets, gate, lp) || hold_launch<C, 5, 512, FAN>(st, a, packets, gate, lp));
     if (took && lp.held) *lp.held = true;
     return took;
 }

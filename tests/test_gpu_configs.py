@@ -174,8 +174,9 @@ def test_c3_ring_through_the_process_group_with_peers_in_pinned_host_memory(env,
     assert errs == [None] * world, errs
     for r in range(world):
         assert torch.equal(base[r].view(torch.int32), want[r].view(torch.int32)), f"rank {r}"
-    for calls, elems, peer_bytes, hbm_bytes, fold_ms, sent in stats:
+    for calls, elems, peer_bytes, hbm_bytes, fold_ms, sent, *legs in stats:
         assert calls == 1 and elems in (27500001, 27499999)
+        assert len(legs) == 5 and all(ms >= 0 for ms in legs) and sum(legs) > 0   # encode, scatter leg, fold, gather leg, casts
         assert peer_bytes == 3 * elems * 2 and fold_ms > 0
         print(f"C3 fold through the backend, peers in pinned host memory: {fold_ms:.2f} ms, "
               f"{peer_bytes / fold_ms / 1e6:.1f} GB/s over PCIe")

@@ -255,3 +255,33 @@ def test_the_gate_follows_the_device_and_the_knobs_override_it(monkeypatch):
     q = K.ReduceQueue(0)
     assert q.hold_model() == (lat, bpt, True), "one measurement per device and process"
     q.close()
+
+
+def test_the_wire_encode_has_a_hold_form_too(env, queues):
+    """fp32 -> bf16 of whole tensors (the first launch of every schedule that sends bf16 copies):
+    reads first, results kept in registers, stores behind the gate -- from three tensors on (on one
+    or two the plain form is as fast or faster).  Bit for bit the oracle's round-to-nearest-even,
+    specials included, on ragged, misaligned segments; the size threshold is off in this queue."""
+    K, L, U, _ = env
+    held, plain = queues
+    rng = np.random.default_rng(9)
+    plan = K.make_plan(BF16, 1, io=L.IO_OWN_FIRST_F32)
+    for counts, takes in (([1], False), ([6_000_001], False), ([300_001, 299_999], False), ([70_003, 5, 123_457], True),
+                          ([2_000_003, 1_500_001, 1_999_999], True), ([1_200_001] * 5 + [7], True)):
+        segs, want, outs = [], [], []
+        for n in counts:
+            off_i, off_o = int(rng.integers(0, 5)), int(rng.integers(0, 5))
+            a = U.rand_values(rng, n + off_i + 4, F32, scale=1e-2, specials=True)
+            t = U.to_dev(a, F32)
+            o = torch.full((n + off_o + 4,), 3.0, dtype=torch.bfloat16, device="cuda")
+            segs.append(K.make_seg(0, o.data_ptr() + 2 * off_o, [t.data_ptr() + 4 * off_i], n))
+            want.append(orc.encode_bf16(np.ascontiguousarray(a[off_i:off_i + n])))
+            outs.append((o, off_o, n, t))
+        torch.cuda.synchronize()
+        before = held.hold_launch_count()
+        held.fold(plan, segs)
+        held.drain()
+        assert held.hold_launch_count() == before + int(takes), f"encode of {counts}: hold form {'not ' if takes else ''}taken"
+        for (o, off, n, _), w in zip(outs, want):
+            assert np.array_equal(U.bits(o[off:off + n]), w), f"encode, hold form, counts {counts}"
+            assert torch.all(o[:off].float() == 3.0) and torch.all(o[off + n:].float() == 3.0), "wrote outside its range"
