@@ -43,8 +43,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 CAL_BYTES = 64 << 20   # size of the calibration copy
 # HBM bytes one C2 fold launch moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by the
-# calibration copy (profiles/c2_fold_hbm_traffic_pmc.txt): 1.004 x the algorithmic bytes.
-C2_MEASURED_TRAFFIC_BYTES = 79_057_166
+# calibration copy (profiles/c2_fold_hbm_traffic_pmc.txt): 1.006 x the algorithmic bytes.
+C2_MEASURED_TRAFFIC_BYTES = 79_121_992
 
 
 def parse():
@@ -59,6 +59,9 @@ def parse():
     ap.add_argument("--timeline", action="store_true",
                     help="instead of the JSON line, print where the time of one C2 launch goes: every block's "
                          "start and end stamps from the measurement build (python -m mccl_amd.build --bench)")
+    ap.add_argument("--host-phases", action="store_true",
+                    help="instead of the JSON line, print where the host's time goes for a C2 bucket through the "
+                         "c10d surface (three native rank threads), phase by phase")
     return ap.parse_args()
 
 
@@ -68,6 +71,10 @@ def main():
         print("bench.py measures one GPU's share of the path; this build runs on a single GPU "
               "(--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
+
+    if args.host_phases:
+        host_phase_report()
+        return
 
     import numpy as np
     import torch
@@ -153,25 +160,61 @@ def main():
             seg_fn(i)
         return qu.graph_end()
 
-    def measure(seg_fn, steps, warmup, wall=False, queue=None):
-        """Untimed warm-up, then exactly `steps` timed steps; returns (device ms, wall ms or None).
-        The warm-up replays the same recorded graph (so at least `warmup` steps, in whole
-        replays, and at least one replay): the first replays of a freshly instantiated graph
-        run about 4 % slower per kernel than later ones, which is a property of the launch
-        path, not of the kernel.  The data stays cold either way: every replay walks all
-        rotating copies again.  Device time: events on the reduce queue around a replay
-        enqueued directly behind the warm-up.  Wall time (`wall=True`): a second replay of
-        the same K steps, bracketed by a drain and a device synchronisation on both sides."""
+    def timed_replays(qu, graph, reps=5):
+        """Median device time (ms) of one replay of `graph`: HIP events on the reduce queue around a
+        replay enqueued directly behind an untimed replay of the same graph."""
+        ts = []
+        for _ in range(reps):
+            qu.graph_launch(graph)
+            qu.timer_begin()
+            qu.graph_launch(graph)
+            ts.append(qu.timer_end())
+        return sorted(ts)[reps // 2]
+
+    # Marks in a kernel trace: a copy of n x 4 KiB (a grid of n x 256 threads of the plain copy kernel)
+    # in front of and behind the headline's timed replays, so that a profile of this program can
+    # tell them from the warm-up around them.
+    mark_buf = torch.zeros(2 * 16 * 4096, dtype=torch.uint8, device="cuda")
+
+    def mark(n):
+        q.copy(mark_buf.data_ptr() + 16 * 4096, mark_buf.data_ptr(), n * 4096)
+
+    def measure(seg_fn, steps, warmup, wall=False, queue=None, reps=5, marks=None):
+        """W untimed warm-up steps, then exactly `steps` timed steps; returns (device ms, wall ms or None).
+        `seg_fn(i)` issues step i.  Device time: two graphs are recorded, one of the W warm-up steps
+        alone and one of the W warm-up steps followed by the `steps` timed ones (W = `warmup`, but at
+        least 10: the first launches behind a graph boundary run slower than the rest).  Each is
+        replayed between a pair of HIP events on the reduce queue; the difference of the two times
+        is the time of steps W+1 .. W+steps: the launches and the gaps between them, with the warm-up
+        and whatever a pair of events and a graph replay add to a bracket (8-11 us, whatever the
+        length of the graph; 0.5 us per step if left inside a bracket of 20 steps) taken out.
+        Medians of `reps` replays.  The data stays cold: every replay walks all rotating copies again.
+        Wall time (`wall=True`): a replay of a graph of the same K steps, bracketed by a drain
+        and a device synchronisation on both sides."""
         qu = queue or q
         torch.cuda.synchronize()  # inputs made by torch ops are complete before the queue reads them
-        gk = record(steps, seg_fn, qu)
-        for _ in range(max(1, -(-warmup // steps))):
-            qu.graph_launch(gk)
-        qu.timer_begin()
-        qu.graph_launch(gk)
-        ms_dev = qu.timer_end()
+        w = max(warmup, min(10, steps))
+        g_warm = record(w, seg_fn, qu)
+        g_all = record(w + steps, seg_fn, qu)
+        # the first replay of a fresh graph is slower still, and a device that has been idle takes
+        # some tens of milliseconds of work to reach its steady clocks: 50 ms of untimed replays
+        t_ready = time.perf_counter() + 0.05
+        while time.perf_counter() < t_ready:
+            for _ in range(4):
+                qu.graph_launch(g_all)
+            qu.drain()
+        if marks:
+            mark(marks[0])
+        ms_all = timed_replays(qu, g_all, reps)
+        if marks:
+            mark(marks[1])
+        ms_dev = ms_all - timed_replays(qu, g_warm, reps)
+        qu.graph_destroy(g_warm)
+        qu.graph_destroy(g_all)
         ms_wall = None
         if wall:
+            gk = record(steps, lambda i: seg_fn(w + i), qu)
+            qu.graph_launch(gk)
             qu.drain()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
@@ -179,7 +222,7 @@ def main():
             qu.drain()
             torch.cuda.synchronize()
             ms_wall = (time.perf_counter() - t0) * 1e3
-        qu.graph_destroy(gk)
+            qu.graph_destroy(gk)
         return ms_dev, ms_wall
 
     cold = lambda i: q.fold(plan, step_segs(i % args.sets, out_tensors=results[i % args.sets]))
@@ -187,8 +230,8 @@ def main():
     if args.timeline:
         timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure, bytes_per_step)
         return
-    cold_dev, cold_wall = measure(cold, args.steps, args.warmup, wall=True)
-    warm_dev, _ = measure(warm, args.steps, args.warmup)
+    cold_dev, cold_wall = measure(cold, args.steps, args.warmup, wall=True, reps=9, marks=(1, 2))
+    warm_dev, _ = measure(warm, args.steps, args.warmup, reps=9, marks=(3, 4))
 
     gbs = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
     kernel_us = cold_dev / args.steps * 1e3
@@ -222,6 +265,10 @@ def main():
              "warm_GBps": round(gbs(bytes_per_step, warm_dev / args.steps), 1),
              "warm_kernel_us": round(warm_dev / args.steps * 1e3, 2),
              "pct_of_hbm_peak_cold": round(100 * achieved / HBM_PEAK_GBS, 2)}
+    # the same launches in single brackets: events around graph replays of 10-160 steps.  A straight
+    # line through (steps, microseconds) has the launch period as its slope and what a graph replay
+    # and the two events add to a bracket as its intercept
+    extra["c2_fold_single_brackets"] = graph_bracket_fit(q, cold, record, np)
 
     if not args.no_extras:
         try:
@@ -261,6 +308,51 @@ def main():
             "cpu_model": cpu_model()}
     result["extra"] = extra
     print(json.dumps(result))
+
+
+def graph_bracket_fit(q, seg_fn, record, np):
+    ks, tot = (10, 20, 40, 80, 160), []
+    for k in ks:
+        g = record(k, seg_fn, q)
+        ts = []
+        for _ in range(5):
+            q.graph_launch(g)
+            q.graph_launch(g)
+            q.timer_begin()
+            q.graph_launch(g)
+            ts.append(q.timer_end() * 1e3)
+        q.graph_destroy(g)
+        tot.append(sorted(ts)[2])
+    slope, icpt = np.linalg.lstsq(np.vstack([ks, np.ones(len(ks))]).T, np.array(tot), rcond=None)[0]
+    return {"us_per_step_by_steps": {str(k): round(t / k, 2) for k, t in zip(ks, tot)},
+            "fit_us_per_step": round(float(slope), 2), "fit_us_per_bracket": round(float(icpt), 1)}
+
+
+def host_phase_report():
+    """Host cost of a C2 bucket through ProcessGroupMCCL, by phase (MCCL_PHASE_STATS=1): eight buckets
+    back to back per round, three ranks as native threads, synchronous and event-based completion."""
+    os.environ["MCCL_PHASE_STATS"] = "1"
+    os.environ.update({"MCCL_ALLREDUCE_ALGO": "butterfly", "MCCL_WIRE_DTYPE": "bf16"})
+    import torch
+    from mccl_amd import _C as CX, workloads as W
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    numel, nb, rounds = W.C2["numel"], 8, 6
+    for mode in ("synchronous", "event-based"):
+        if mode == "event-based":
+            os.environ["MCCL_ALLREDUCE_ASYNC"] = "1"
+        else:
+            os.environ.pop("MCCL_ALLREDUCE_ASYNC", None)
+        CX._allreduce_rate(3, numel, nb, 2)   # first rounds: kernels loaded, graphs recorded
+        CX._phase_stats(True)
+        us = CX._allreduce_rate(3, numel, nb, rounds)
+        st = CX._phase_stats(True)
+        print(f"{mode} completion: best round, us per bucket, by rank: {[round(x, 1) for x in us]}")
+        print(f"  {'phase':15s} {'calls':>6s} {'mean us':>9s} {'us per bucket, all 3 ranks together':>38s}")
+        for k, (calls, tot) in st.items():
+            if calls:
+                print(f"  {k:15s} {calls:6d} {tot / calls:9.2f} {tot / (nb * rounds):38.2f}")
 
 
 def cpu_model() -> str:
@@ -310,9 +402,12 @@ def timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure,
     pr("instruction, at a second point, and after its last store was issued.  16 consecutive launches (cold = rotating 8")
     pr("copies of the workload, 944 MB + 629 MB of results) are recorded into one HIP graph; figures are means over")
     pr("launches 3..15 of its 4th replay.  All times in microseconds.")
-    pr("  hold form  (the default for this launch): 1023 blocks of 512 threads, ONE generation; every lane issues the loads")
+    lat_ticks, bpt, measured = q.hold_model()
+    pr("  hold form  (the default for this launch): 1020 blocks of 512 threads, ONE generation; every lane issues the loads")
     pr("             of its four packets at once, keeps the results in registers and stores them when the gate opens")
-    pr("             (40 ticks + bytes read / 71,000 per tick after its block started).  Second stamp: the block has its data.")
+    pr(f"             ({lat_ticks} ticks + bytes read / {bpt:,} per tick after its block started; the rate was "
+       f"{'measured on this device' if measured else 'taken from the built-in default'}).")
+    pr("             Second stamp: the block has its data.")
     pr("  plain form (mcclx_set_hold(ctx, 0); every launch too large for one generation): 3201 blocks, one per 8 KiB tile of")
     pr("             a chunk, loads then stores.  Second stamp: the block has its kernel arguments.")
 
@@ -803,6 +898,14 @@ def extras(args, q, K, H, L, W, torch, np, tensors, wires, chunks, plan, step_se
         out[f"c2_allreduce_{name}_in_graph_us_per_bucket"] = round(ms / steps * 1e3, 1)
     out["c2_allreduce_direct_in_graph_GBps"] = round(gbs(world * numel * 8, ms / steps), 1)
     ws.free()
+    # its ceiling: the plain copy kernel over the same footprint (78.6 MB in, 78.6 MB out, cold)
+    half = world * numel * 4
+    pool = torch.randint(0, 256, (8 * half,), dtype=torch.uint8, device="cuda")
+    ms, _ = measure(lambda i: q.copy(pool.data_ptr() + (2 * (i % 4) + 1) * half, pool.data_ptr() + 2 * (i % 4) * half, half),
+                    steps, warm)
+    out["c2_allreduce_direct_footprint_plain_copy_us"] = round(ms / steps * 1e3, 1)
+    out["c2_allreduce_direct_footprint_plain_copy_GBps"] = round(gbs(2 * half, ms / steps), 1)
+    del pool
 
     # C1: ring, 2 ranks, 1 Mi fp32, SUM: one k=2 fold per chunk
     x = [torch.randn(W.C1["numel"], device="cuda") for _ in range(2 * 8)]

@@ -78,7 +78,7 @@ struct LaunchParams {
     bool* held = nullptr;              // set when the launch took that form (diagnostic)
     uint64_t hold_min_read_bytes = 0;
     uint32_t hold_latency_ticks = 40;
-    uint32_t hold_bytes_per_tick = 71000;
+    uint32_t hold_bytes_per_tick = 72000;
 };
 // Plans that have a fan-out form: sums with per-step rounding, 2..7 operands.
 bool fan_plan_ok(const PlanKey& key);

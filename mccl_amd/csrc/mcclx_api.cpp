@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <atomic>
+#include <chrono>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -78,7 +79,7 @@ struct mcclx_ctx {
     bool validate = false;
     // reads-then-writes launches (LaunchParams): least bytes read, and the gate's model
     uint64_t hold_min_read_bytes = 10ull << 20;
-    uint32_t hold_latency_ticks = 40, hold_bytes_per_tick = 71000;  // in ticks of 100 MHz
+    uint32_t hold_latency_ticks = 40, hold_bytes_per_tick = 72000;  // in ticks of 100 MHz
     uint32_t wall_khz = 100000;                                      // the device's wall clock
     bool hold_measured = false;        // the gate's rate was measured on this device (not the default)
     std::atomic<bool> hold_enabled{true};  // a completer thread may switch it while ranks launch
@@ -523,26 +524,27 @@ int fold_impl(mcclx_ctx* ctx, const mcclx_plan* plan, const mcclx_seg* segs, uin
 // latency + bytes read / rate -- has one constant that differs from part to part and from
 // one memory configuration to the next: the rate at which a launch's reads come in.  It is
 // measured once per device and process, when the first context is made: read-only launches of
-// two sizes over a scratch buffer larger than the Infinity Cache (so they read HBM, as a
-// gradient bucket does), the difference of their times over the difference of their sizes.
-// On MI355X the best gate of a 25 MiB bucket, swept, sits at 0.995 of the rate this probe
-// measures (a fold's reads come in a little slower than a single stream's: several address
-// streams, the arithmetic of the late waves), and that ratio is what carries over to
-// another device.
+// two sizes (24 and 96 MiB) over a scratch buffer larger than the Infinity Cache (so they read
+// HBM, as a gradient bucket does), the difference of their times over the difference of their
+// sizes, after 20 ms of the same probe (a device that has been idle needs that long to reach its
+// steady clocks); the figure repeats within 1 % from process to process.  On MI355X the best gate
+// of a 25 MiB bucket, swept, sits at 760-775 ticks after a block's start, flat within 0.05 us
+// across that range, 0.2 us worse 3 % earlier and 0.15 us worse 6 % later: 1.005 of the rate
+// this probe measures, and that ratio is what carries over to another device.
 // MCCLX_HOLD_CALIBRATE=0 keeps the defaults; the MCCLX_HOLD_* knobs override either.
 struct HoldModel {
     uint32_t latency_ticks = 40;      // ticks of 100 MHz
-    uint32_t bytes_per_tick = 71000;  // per tick of 100 MHz
+    uint32_t bytes_per_tick = 72000;  // per tick of 100 MHz
     bool measured = false;
 };
-constexpr double kHoldGateRatio = 0.995;
+constexpr double kHoldGateRatio = 1.005;
 
 HoldModel measure_hold_model() {  // the device is current
     HoldModel m;
     if (const char* v = getenv("MCCLX_HOLD_CALIBRATE"))
         if (v[0] == '0') return m;
-    constexpr size_t kBig = 48u << 20, kSmall = 24u << 20;
-    constexpr int kCopies = 8;  // 384 MiB: more than the 256 MiB Infinity Cache
+    constexpr size_t kBig = 96u << 20, kSmall = 24u << 20;  // the launches that hold read 10-100 MB
+    constexpr int kCopies = 4;  // 384 MiB: more than the 256 MiB Infinity Cache
     char* buf = nullptr;
     hipStream_t st = nullptr;
     hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -562,10 +564,18 @@ HoldModel measure_hold_model() {  // the device is current
     bool ok = true;
     for (int i = 0; i < kCopies && ok; ++i)  // a payload of mixed bits (zero-filled memory reads faster)
         ok = mcclx::launch_stream_probe(st, buf + (size_t)i * kBig, kBig, true) == hipSuccess;
-    auto timed = [&](size_t nbytes) -> double {  // microseconds per launch, best of three rounds
+    // A device that has been idle takes some tens of milliseconds of work to reach its steady
+    // clocks, and the first context of a process is often its first work: 20 ms of the probe first.
+    for (const auto until = std::chrono::steady_clock::now() + std::chrono::milliseconds(20);
+         ok && std::chrono::steady_clock::now() < until;) {
+        for (int i = 0; i < 16 && ok; ++i)
+            ok = mcclx::launch_stream_probe(st, buf + (size_t)(i % kCopies) * kBig, kBig, false) == hipSuccess;
+        ok = ok && hipStreamSynchronize(st) == hipSuccess;
+    }
+    auto timed = [&](size_t nbytes) -> double {  // microseconds per launch, best of five rounds
         double best = 1e30;
         for (int round = 0; round < 5 && ok; ++round) {
-            constexpr int kReps = 24;
+            constexpr int kReps = 32;
             for (int i = 0; i < 4 && ok; ++i)
                 ok = mcclx::launch_stream_probe(st, buf + (size_t)(i % kCopies) * kBig, nbytes, false) == hipSuccess;
             ok = ok && hipEventRecord(e0, st) == hipSuccess;

@@ -165,7 +165,7 @@ uint64_t mcclx_hold_launch_count(mcclx_ctx*) { return 0; }
 int mcclx_set_hold(mcclx_ctx*, int) { return MCCLX_OK; }
 int mcclx_hold_model(mcclx_ctx*, uint32_t* a, uint32_t* b) {
     if (a) *a = 40;
-    if (b) *b = 71000;
+    if (b) *b = 72000;
     return 0;
 }
 
