@@ -523,7 +523,7 @@ def timeline_report(args, q, K, L, torch, np, plan, step_segs, results, measure,
     ms, _ = measure(lambda i: q.probe_stream(probe.data_ptr(), 16 * 256, False), steps, args.warmup)
     empty_us = ms / steps * 1e3
     pr("")
-    pr(f"[the same launches without stamps, {steps} per graph replay, HIP events around the replay; cold]")
+    pr(f"[the same launches without stamps, {steps} timed steps behind {max(args.warmup, min(10, steps))} warm-up steps in one graph, HIP events, the warm-up graph's time subtracted; cold]")
     pr(f"  C2 fold (52.4 MB read + 26.2 MB written), hold form {fold_us:6.2f} us per launch = {gbs(fp, fold_us * 1e-3):6.0f} GB/s = {gbs(fp, fold_us * 1e-3) / 80:5.1f} % of 8 TB/s")
     pr(f"  the same, plain form                                {plain_us:6.2f} us per launch = {gbs(fp, plain_us * 1e-3):6.0f} GB/s = {gbs(fp, plain_us * 1e-3) / 80:5.1f} % of 8 TB/s")
     for name, us, g in lines:
