@@ -702,10 +702,8 @@ __global__ void __launch_bounds__(kHoldBlock) fold_few_hold_kernel(FewArgs a, ui
 // schedule that sends bf16 copies; ten 16-byte packets per lane cover three 25 MiB tensors).
 template <class C>
 constexpr bool kHoldEncode = C::K == 1 && C::IO == MCCLX_IO_OWN_FIRST_F32 && C::ACC == MCCLX_ACC_STEP;
-#ifndef MCCLX_HOLD_ENCODE_EARLY
-#define MCCLX_HOLD_ENCODE_EARLY 105
-#endif
-constexpr uint64_t kHoldEncodeEarlyPct = MCCLX_HOLD_ENCODE_EARLY;
+constexpr uint64_t kHoldEncodeEarlyPct = 105;  // the encode's gate: the model's rate taken 5 % higher
+constexpr uint64_t kHoldFanLatePct = 97;       // a fan-out fold's gate: the model's rate taken 3 % lower
 template <class C>
 constexpr bool kHoldPlan = ((C::K >= 2 && C::K <= 4) || kHoldEncode<C>) && C::OP == MCCLX_SUM &&
                            C::ACC == MCCLX_ACC_STEP && C::TOPO == MCCLX_TOPO_FOLD;
@@ -763,7 +761,7 @@ static bool try_hold(hipStream_t st, FewArgs& a, uint64_t maxc, const LaunchPara
     // fold that writes as much as it reads (fan-out), with them a little late (the one-launch
     // allreduce of a 25 MiB bucket: 27.3 us at the fold's gate, 26.7 us 2-4 % later, 27.1 us 8 % later)
     if constexpr (kHoldEncode<C>) ticks = lp.hold_latency_ticks + read_bytes * 100 / (lp.hold_bytes_per_tick * kHoldEncodeEarlyPct);
-    if constexpr (FAN) ticks = lp.hold_latency_ticks + read_bytes * 100 / (lp.hold_bytes_per_tick * 97ull);
+    if constexpr (FAN) ticks = lp.hold_latency_ticks + read_bytes * 100 / (lp.hold_bytes_per_tick * kHoldFanLatePct);
     const uint32_t gate = ticks > 100000 ? 100000u : (uint32_t)ticks;  // a millisecond at most
     const uint64_t packets = (maxc + C::E - 1) / C::E;
     // A fold with one output takes four packets per lane if that covers it.  One that writes as
