@@ -285,3 +285,47 @@ def test_the_wire_encode_has_a_hold_form_too(env, queues):
         for (o, off, n, _), w in zip(outs, want):
             assert np.array_equal(U.bits(o[off:off + n]), w), f"encode, hold form, counts {counts}"
             assert torch.all(o[:off].float() == 3.0) and torch.all(o[off + n:].float() == 3.0), "wrote outside its range"
+
+
+@pytest.mark.parametrize("with_out,with_wire,scaled", [(True, False, False), (True, True, True), (False, True, True), (True, True, False)])
+def test_one_operand_plans_in_the_hold_form_match_the_plain_form(env, queues, with_out, with_wire, scaled):
+    """The encode's plan (one fp32 operand, rounded to bf16) with any of its outputs -- the fp32
+    form of the rounded value, the bf16 form, both -- and with a scale: the hold form writes what
+    the plain form writes, bit for bit, and nothing outside, on ragged segments that include an
+    empty one and one shorter than the head peel."""
+    K, L, U, _ = env
+    held, plain = queues
+    rng = np.random.default_rng(77 + 4 * with_out + 2 * with_wire + scaled)
+    plan = K.make_plan(BF16, 1, io=L.IO_OWN_FIRST_F32, scale_mode=L.SCALE_VIEW if scaled else L.SCALE_NONE, scale=1.0 / 3)
+    for counts in ([70_003, 0, 123_457], [3, 500_001, 17, 250_000], [1_000_003] * 3):
+        ins = []
+        for n in counts:
+            off = int(rng.integers(0, 5))
+            a = U.rand_values(rng, n + off + 4, F32, scale=1e-2, specials=True)
+            ins.append((U.to_dev(a, F32), off, n))
+        got = []
+        for q in (held, plain):
+            outs, segs = [], []
+            for t, off, n in ins:
+                oo, ow = int(rng.integers(0, 5)), int(rng.integers(0, 5))
+                o = torch.full((n + oo + 4,), 3.0, device="cuda") if with_out else None
+                w = torch.full((n + ow + 4,), 3.0, dtype=torch.bfloat16, device="cuda") if with_wire else None
+                segs.append(K.make_seg(o.data_ptr() + 4 * oo if with_out else 0, w.data_ptr() + 2 * ow if with_wire else 0,
+                                       [t.data_ptr() + 4 * off], n))
+                outs.append((o, oo, w, ow, n))
+            torch.cuda.synchronize()
+            before = q.hold_launch_count()
+            q.fold(plan, segs)
+            q.drain()
+            assert q.hold_launch_count() == before + (1 if q is held else 0)
+            for o, oo, w, ow, n in outs:
+                if with_out:
+                    assert torch.all(o[:oo] == 3.0) and torch.all(o[oo + n:] == 3.0), "wrote outside its range"
+                if with_wire:
+                    assert torch.all(w[:ow].float() == 3.0) and torch.all(w[ow + n:].float() == 3.0), "wrote outside its range"
+            got.append([(o[oo:oo + n].clone() if with_out else None, w[ow:ow + n].clone() if with_wire else None) for o, oo, w, ow, n in outs])
+        for (ho, hw), (po, pw) in zip(*got):
+            if with_out:
+                assert torch.equal(ho.view(torch.int32), po.view(torch.int32)), f"fp32 output, counts {counts}"
+            if with_wire:
+                assert torch.equal(hw.view(torch.int16), pw.view(torch.int16)), f"bf16 output, counts {counts}"
