@@ -703,7 +703,7 @@ __global__ void __launch_bounds__(kHoldBlock) fold_few_hold_kernel(FewArgs a, ui
 template <class C>
 constexpr bool kHoldEncode = C::K == 1 && C::IO == MCCLX_IO_OWN_FIRST_F32 && C::ACC == MCCLX_ACC_STEP;
 constexpr uint64_t kHoldEncodeEarlyPct = 105;  // the encode's gate: the model's rate taken 5 % higher
-constexpr uint64_t kHoldFanLatePct = 97;       // a fan-out fold's gate: the model's rate taken 3 % lower
+constexpr uint64_t kHoldFanLatePct = 97;       // a fan-out fold at five packets per lane: the model's rate taken 3 % lower
 template <class C>
 constexpr bool kHoldPlan = ((C::K >= 2 && C::K <= 4) || kHoldEncode<C>) && C::OP == MCCLX_SUM &&
                            C::ACC == MCCLX_ACC_STEP && C::TOPO == MCCLX_TOPO_FOLD;
@@ -757,22 +757,23 @@ static bool try_hold(hipStream_t st, FewArgs& a, uint64_t maxc, const LaunchPara
     if constexpr (kHoldEncode<C>)
         if (a.nseg < 3 || read_bytes < lp.hold_min_read_bytes * 9 / 5) return false;
     uint64_t ticks = lp.hold_latency_ticks + read_bytes / lp.hold_bytes_per_tick;
-    // the encode writes half of what it reads and does best with its stores a little early; a
-    // fold that writes as much as it reads (fan-out), with them a little late (the one-launch
-    // allreduce of a 25 MiB bucket: 27.3 us at the fold's gate, 26.7 us 2-4 % later, 27.1 us 8 % later)
+    // the encode writes half of what it reads and does best with its stores a little early
     if constexpr (kHoldEncode<C>) ticks = lp.hold_latency_ticks + read_bytes * 100 / (lp.hold_bytes_per_tick * kHoldEncodeEarlyPct);
-    if constexpr (FAN) ticks = lp.hold_latency_ticks + read_bytes * 100 / (lp.hold_bytes_per_tick * kHoldFanLatePct);
+    uint32_t gate5 = 0;  // a fan-out fold at five packets per lane (fewer waves, more loads each): its reads take 3 % longer
+    if constexpr (FAN) {
+        const uint64_t t5 = lp.hold_latency_ticks + read_bytes * 100 / (lp.hold_bytes_per_tick * kHoldFanLatePct);
+        gate5 = t5 > 100000 ? 100000u : (uint32_t)t5;
+    }
     const uint32_t gate = ticks > 100000 ? 100000u : (uint32_t)ticks;  // a millisecond at most
     const uint64_t packets = (maxc + C::E - 1) / C::E;
-    // A fold with one output takes four packets per lane if that covers it.  One that writes as
-    // much as it reads (fan-out) does better with five and fewer waves: the one-launch allreduce
-    // of a 25 MiB bucket 26.5 us against 27.6 us (of a 16 MiB bucket 17.4 against 17.2 us).
+    // Four packets per lane if that covers the launch, five otherwise.  (The one-launch allreduce of a
+    // 25 MiB bucket, which writes as much as it reads: 26.2 us at four, each form at its best gate,
+    // 26.7 us at five.)
     bool took;
     if constexpr (kHoldEncode<C>)
         took = hold_launch<C, 10, 512, false>(st, a, packets, gate, lp);
     else
-        took = FAN ? (hold_launch<C, 5, 512, FAN>(st, a, packets, gate, lp) || hold_launch<C, 4, 512, FAN>(st, a, packets, gate, lp))
-                   : (hold_launch<C, 4, 512, FAN>(st, a, packets, gate, lp) || hold_launch<C, 5, 512, FAN>(st, a, packets, gate, lp));
+        took = hold_launch<C, 4, 512, FAN>(st, a, packets, gate, lp) || hold_launch<C, 5, 512, FAN>(st, a, packets, FAN ? gate5 : gate, lp);
     if (took && lp.held) *lp.held = true;
     return took;
 }
