@@ -543,7 +543,7 @@ HoldModel measure_hold_model() {  // the device is current
     HoldModel m;
     if (const char* v = getenv("MCCLX_HOLD_CALIBRATE"))
         if (v[0] == '0') return m;
-    constexpr size_t kBig = 96u << 20, kSmall = 24u << 20;  // the launches that hold read 10-100 MB
+    constexpr size_t kBig = 96u << 20, kMid = 60u << 20, kSmall = 24u << 20;  // the launches that hold read 10-100 MB
     constexpr int kCopies = 4;  // 384 MiB: more than the 256 MiB Infinity Cache
     char* buf = nullptr;
     hipStream_t st = nullptr;
@@ -588,13 +588,24 @@ HoldModel measure_hold_model() {  // the device is current
         }
         return best;
     };
-    const double t_small = timed(kSmall), t_big = timed(kBig);
+    const double t_small = timed(kSmall), t_mid = timed(kMid), t_big = timed(kBig);
     cleanup();
-    if (!ok || !(t_big > t_small)) return m;
+    if (!ok || !(t_mid > t_small) || !(t_big > t_mid)) return m;
     const double probe_rate = (double)(kBig - kSmall) / ((t_big - t_small) * 100.0);  // bytes per 10 ns
     const double rate = probe_rate * kHoldGateRatio;
-    // a device busy with someone else's work while this ran gives nonsense: keep the default then
-    if (rate < 0.5 * m.bytes_per_tick || rate > 2.0 * m.bytes_per_tick) return m;
+    // A device busy with someone else's work while this ran, or a tool that stretches launches and
+    // event times (a profiler: 111,000 B per tick was once "measured" under one), gives nonsense:
+    // the two halves of the size range must agree on the rate within 15 % (undisturbed, the lower half
+    // reads 5-8 % faster than the upper; under a profiler the shortest launch takes twice its time and
+    // the halves differ by a factor of two to four), and the rate must be one a part of this family
+    // can have; otherwise the built-in constants stay.
+    const double lower = (double)(kMid - kSmall) / (t_mid - t_small), upper = (double)(kBig - kMid) / (t_big - t_mid);
+    if (const char* v = getenv("MCCLX_HOLD_CALIBRATE"))
+        if (v[0] == '2')  // say what was measured
+            fprintf(stderr, "[mcclx] gate calibration: %.2f / %.2f / %.2f us for 24 / 60 / 96 MiB read; %.0f B per 10 ns "
+                            "(lower half %.0f, upper half %.0f)\n", t_small, t_mid, t_big, probe_rate, lower / 100.0, upper / 100.0);
+    if (lower > 1.15 * upper || upper > 1.15 * lower) return m;
+    if (rate < 0.6 * m.bytes_per_tick || rate > 1.4 * m.bytes_per_tick) return m;
     m.bytes_per_tick = (uint32_t)rate;
     m.measured = true;
     return m;
