@@ -42,3 +42,11 @@ def test_the_headline_range_in_the_readme_covers_the_committed_measurements():
     # and the fraction of the peak that goes with it
     pct = re.search(r"\((\d+)–(\d+) %\s+of the 8 TB/s HBM peak", readme)
     assert pct and abs(78.6432 / hi / 8 * 100 - int(pct.group(1))) <= 1 and abs(78.6432 / lo / 8 * 100 - int(pct.group(2))) <= 1
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    """This build measures one GPU's share of the path: `bench.py --gpus N` with N above 1 says so and exits."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 2 and "single GPU" in r.stderr and r.stdout.strip() == ""
