@@ -135,9 +135,11 @@ private:
     std::mutex mu_;
     std::condition_variable cv_;
     std::vector<Contribution> slots_;
-    int arrived_ = 0;
-    std::atomic<uint64_t> generation_{0};  // written under mu_; read without it while a waiter spins
-    std::exception_ptr last_error_;
+    static constexpr int kCountBits = 16;
+    static constexpr uint64_t kCountMask = (1ull << kCountBits) - 1;
+    std::atomic<uint64_t> state_{0};       // generation << 16 | ranks that have arrived for it; the last arrival moves
+                                           // the generation on when its work is done, the others poll it
+    std::exception_ptr last_error_;        // of the collective that just ended: written before the generation moves on
     std::atomic<bool> broken_{false};
     const int spin_us_;                    // how long a waiter polls before it sleeps (MCCL_MEET_SPIN_US)
 

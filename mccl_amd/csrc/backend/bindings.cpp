@@ -258,19 +258,22 @@ std::tuple<bool, bool, std::string> work_probe(const std::string& mode, int wait
 }
 
 // N threads meet `rounds` times in a LocalMesh; rank `absent` (if >= 0) never
-// shows up, rank `thrower` makes the leader throw.  Returns per-rank messages.
-std::vector<std::string> mesh_probe(int world, int rounds, int absent, int timeout_ms, bool leader_throws) {
+// shows up -- or shows up `late_ms` milliseconds after the others, if that is given --,
+// `leader_throws` makes the leader throw.  Returns per-rank messages; a leader that ran
+// although a rank had already left with a timeout shows as a count in the late rank's message.
+std::vector<std::string> mesh_probe(int world, int rounds, int absent, int timeout_ms, bool leader_throws, int late_ms) {
     auto mesh = mccl::LocalMesh::create(mccl::LocalMesh::fresh_key(), world);
     std::vector<std::string> out(static_cast<size_t>(world));
     std::vector<std::thread> ts;
     std::atomic<int> leader_runs{0};
     for (int r = 0; r < world; ++r) {
-        if (r == absent) {
+        if (r == absent && late_ms < 0) {
             out[static_cast<size_t>(r)] = "absent";
             continue;
         }
         ts.emplace_back([&, r] {
             try {
+                if (r == absent) std::this_thread::sleep_for(std::chrono::milliseconds(late_ms));
                 for (int i = 0; i < rounds; ++i) {
                     mccl::Contribution c;
                     c.kind = 100 + i;
@@ -493,6 +496,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("_test_peer_wire", &peer_wire_probe, py::arg("mode"), py::arg("world") = 3, py::arg("rounds") = 6,
           py::arg("timeout_ms") = 5000, py::call_guard<py::gil_scoped_release>());
     m.def("_test_mesh", &mesh_probe, py::arg("world"), py::arg("rounds") = 3, py::arg("absent") = -1,
-          py::arg("timeout_ms") = 2000, py::arg("leader_throws") = false,
+          py::arg("timeout_ms") = 2000, py::arg("leader_throws") = false, py::arg("late_ms") = -1,
           py::call_guard<py::gil_scoped_release>());
 }

@@ -107,6 +107,17 @@ def test_mesh_times_out_when_a_rank_is_missing(CX):
     assert all(o.startswith("[MCCL] Timeout: ") for i, o in enumerate(out) if i != 1)
 
 
+def test_a_rank_that_arrives_after_its_peers_gave_up_finds_the_mesh_broken(CX):
+    """The peers' arrivals were taken back when their wait timed out: the late rank does not become
+    the leader of a collective whose other members have left (their buffers may be gone)."""
+    out = CX._test_mesh(3, 1, 1, 100, False, 400)
+    assert out[0].startswith("[MCCL] Timeout: ") and out[2].startswith("[MCCL] Timeout: ")
+    assert "broken" in out[1] or out[1].startswith("[MCCL] Timeout: "), out
+    assert not out[1].startswith("ok"), "the leader ran with contributions of ranks that had left"
+    # arriving while the others still wait is fine, however close to their limit
+    assert CX._test_mesh(3, 2, 1, 2000, False, 300) == ["ok:2"] * 3
+
+
 def test_mesh_leader_error_reaches_every_rank(CX):
     assert CX._test_mesh(3, 2, -1, 5000, True) == ["[MCCL] leader failed"] * 3
 

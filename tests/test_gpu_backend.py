@@ -335,6 +335,49 @@ def test_divergent_argument_error_fails_every_rank_at_once(CX):
         assert ok == [6.0] * 5
 
 
+@pytest.mark.parametrize("spin_us", [None, "0", "1"])
+def test_synchronous_allreduce_returns_with_the_result_whichever_way_it_drains(CX, U, monkeypatch, spin_us):
+    """The synchronous allreduce leaves its drain when a word written behind the launch arrives in
+    pinned host memory (the default), after a blocking drain (MCCL_DRAIN_SPIN_US=0), or after a
+    blocking drain because the word did not come within the time allowed (1 us: a 25 MiB bucket
+    takes longer).  Either way the tensors hold the oracle's bits when it returns: read by a kernel
+    on the rank's stream, and by a copy to the host, at once."""
+    if spin_us is None:
+        monkeypatch.delenv("MCCL_DRAIN_SPIN_US", raising=False)
+    else:
+        monkeypatch.setenv("MCCL_DRAIN_SPIN_US", spin_us)
+    monkeypatch.setenv("MCCL_ALLREDUCE_ALGO", "butterfly")
+    monkeypatch.setenv("MCCL_WIRE_DTYPE", "bf16")
+    monkeypatch.delenv("MCCL_ALLREDUCE_ASYNC", raising=False)
+    world = 3
+    sizes = [6_553_600, 33, 1_000_003, 6_553_600, 70_001]
+    rng = np.random.default_rng(41)
+    xs = [[(rng.standard_normal(n) * 1e-3).astype(np.float32) for _ in range(world)] for n in sizes]
+
+    def fn(r, pg):
+        got = []
+        for x in xs:
+            t = U.to_dev(x[r], F32)
+            torch.cuda.current_stream().synchronize()
+            o = dist.AllreduceOptions(); o.reduceOp = dist.ReduceOp.AVG
+            w = pg.allreduce([t], o)
+            assert w.is_completed() and w.is_success()
+            doubled = t * 2                       # a kernel on the rank's stream, straight away
+            host = t.cpu()                        # and a copy to the host
+            got.append((host, doubled.cpu()))
+        return got
+
+    out, errs = run_ranks(CX, world, fn)
+    assert errs == [None] * world, errs
+    for i, n in enumerate(sizes):
+        want = [x.copy() for x in xs[i]]
+        rc, used = orc.pg_allreduce(want, F32, AVG, wire_bf16=True, env_algo="butterfly", threads=orc.max_threads())
+        assert rc == 0 and used == BUTTERFLY
+        for r in range(world):
+            U.assert_same_bits(out[r][i][0], want[r], F32, f"bucket {i} rank {r}")
+            assert torch.equal(out[r][i][1], out[r][i][0] * 2)
+
+
 @pytest.mark.parametrize("queues,direct", [(1, True), (2, True), (2, False)])
 def test_allreduce_event_based_completion_and_bucket_coalescing(CX, U, monkeypatch, queues, direct):
     """MCCL_ALLREDUCE_ASYNC=1: allreduce returns a pending Work, wait() orders the caller's
