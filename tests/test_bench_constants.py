@@ -25,7 +25,7 @@ def test_traffic_constant_equals_the_profile_total():
 def test_the_headline_range_in_the_readme_covers_the_committed_measurements():
     """README.md quotes the headline launch as a range of microseconds; the figures it stands for are
     the unprofiled runs quoted in the kernel-trace profile (the driver's command line and the
-    default step count) and the headline row of DESIGN.md's measured table."""
+    default step count) and the headline row of the design document's measured table."""
     readme = open(os.path.join(ROOT, "README.md")).read()
     m = re.search(r"runs in (\d+\.\d+)–(\d+\.\d+) µs per launch", readme)
     assert m, "README.md no longer states the headline as a range"
@@ -36,7 +36,7 @@ def test_the_headline_range_in_the_readme_covers_the_committed_measurements():
     assert len(runs) == 2, "the profile quotes one unprofiled run per command line"
     design = open(os.path.join(ROOT, "DESIGN.md")).read()
     row = re.search(r"\*\*C2 fused fold, cold \(headline\)\*\* \| \*\*(\d+\.\d+) µs[^|]*\| \*\*(\d+\.\d+) µs", design)
-    assert row, "DESIGN.md's measured table has no headline row"
+    assert row, "the design document's measured table has no headline row"
     for us in runs + [float(row.group(1)), float(row.group(2))]:
         assert lo <= us <= hi, (us, lo, hi)
     # and the fraction of the peak that goes with it
