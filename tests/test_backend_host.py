@@ -118,6 +118,20 @@ def test_a_rank_that_arrives_after_its_peers_gave_up_finds_the_mesh_broken(CX):
     assert CX._test_mesh(3, 2, 1, 2000, False, 300) == ["ok:2"] * 3
 
 
+def test_a_rank_arriving_as_its_peers_time_out_is_served_by_all_or_by_none(CX):
+    """The late rank arrives at about the moment the others' wait runs out.  Whichever way each round
+    falls, it falls one way for everybody: either the collective ran with all three (a rank that
+    could not take its arrival back any more waited for the leader), or nobody's did."""
+    all_ok = none_ok = 0
+    for i in range(150):
+        out = CX._test_mesh(3, 1, i % 3, 4, False, 4)
+        oks = [o.startswith("ok") for o in out]
+        assert all(oks) or not any(oks), out
+        all_ok += all(oks)
+        none_ok += not any(oks)
+    assert all_ok + none_ok == 150
+
+
 def test_mesh_leader_error_reaches_every_rank(CX):
     assert CX._test_mesh(3, 2, -1, 5000, True) == ["[MCCL] leader failed"] * 3
 
