@@ -440,14 +440,22 @@ struct ProcessGroupMCCL::Shared : std::enable_shared_from_this<ProcessGroupMCCL:
             w.spin_us = e ? std::strtol(e, nullptr, 10) : 1000;
             if (w.spin_us < 0) w.spin_us = 0;
             if (w.spin_us > 0) {
-                check_rc(mcclx_host_alloc(ctx, 4096, &w.host, &w.alias));
-                auto* h = static_cast<uint32_t*>(w.host);
-                h[0] = 0;
-                for (uint32_t i = 0; i < DrainWord::kNumbers; ++i) h[256 + i] = i + 1;
-                w.numbers = dev::empty_bytes(4 * DrainWord::kNumbers, device);
-                order_after_allocator(ctx, device);
-                check_rc(mcclx_copy(ctx, w.numbers.data_ptr(), static_cast<char*>(w.alias) + 1024, 4 * DrainWord::kNumbers));
-                check_rc(mcclx_queue_drain(ctx));
+                try {
+                    check_rc(mcclx_host_alloc(ctx, 4096, &w.host, &w.alias));
+                    auto* h = static_cast<uint32_t*>(w.host);
+                    h[0] = 0;
+                    for (uint32_t i = 0; i < DrainWord::kNumbers; ++i) h[256 + i] = i + 1;
+                    w.numbers = dev::empty_bytes(4 * DrainWord::kNumbers, device);
+                    order_after_allocator(ctx, device);
+                    check_rc(mcclx_copy(ctx, w.numbers.data_ptr(), static_cast<char*>(w.alias) + 1024, 4 * DrainWord::kNumbers));
+                    check_rc(mcclx_queue_drain(ctx));
+                } catch (const std::exception& e) {  // no pinned memory to be had: the blocking drain serves
+                    MCCL_WARN("the synchronous allreduce keeps the blocking drain: %s", e.what());
+                    if (w.host) (void)mcclx_host_free(ctx, w.host);
+                    w.host = w.alias = nullptr;
+                    w.numbers = at::Tensor();
+                    w.spin_us = 0;
+                }
             }
         }
         if (w.spin_us == 0) {
