@@ -44,7 +44,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 CAL_BYTES = 64 << 20   # size of the calibration copy
 # HBM bytes one C2 fold launch moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by the
 # calibration copy (profiles/c2_fold_hbm_traffic_pmc.txt): 1.006 x the algorithmic bytes.
-C2_MEASURED_TRAFFIC_BYTES = 79_073_095
+C2_MEASURED_TRAFFIC_BYTES = 79_070_677
 
 
 def parse():
