@@ -179,6 +179,8 @@ def main():
     def mark(n):
         q.copy(mark_buf.data_ptr() + 16 * 4096, mark_buf.data_ptr(), n * 4096)
 
+    single_bracket = {}
+
     def measure(seg_fn, steps, warmup, wall=False, queue=None, reps=5, marks=None):
         """W untimed warm-up steps, then exactly `steps` timed steps; returns (device ms, wall ms or None).
         `seg_fn(i)` issues step i.  Device time: two graphs are recorded, one of the W warm-up steps
@@ -214,6 +216,9 @@ def main():
         ms_wall = None
         if wall:
             gk = record(steps, lambda i: seg_fn(w + i), qu)
+            # the same K steps in ONE pair of events (a replay behind an untimed replay): what the
+            # subtraction above takes out stays in, 7-11 us per bracket
+            single_bracket["ms"] = timed_replays(qu, gk, reps)
             qu.graph_launch(gk)
             qu.drain()
             torch.cuda.synchronize()
@@ -257,7 +262,11 @@ def main():
                    "algorithmic_bytes_per_step": bytes_per_step, "parity_vs_oracle_bit_exact": parity},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": C2_MEASURED_TRAFFIC_BYTES,
-                     "kernel": "fold_few_hold_kernel<bf16, own-first fp32, k=3; 4 packets per lane, 512-lane blocks>", "kernel_us": round(kernel_us, 2)},
+                     "kernel": "fold_few_hold_kernel<bf16, own-first fp32, k=3; 4 packets per lane, 512-lane blocks>", "kernel_us": round(kernel_us, 2),
+                     "method": "HIP events on the reduce queue; time of a graph of W warm-up + K timed launches minus time of a graph "
+                               "of the W warm-up launches alone (W >= 10), medians of 9 replays each, behind 50 ms of untimed replays",
+                     "kernel_us_single_bracket": round(single_bracket["ms"] / args.steps * 1e3, 2),
+                     "frac_single_bracket": round(gbs(bytes_per_step, single_bracket["ms"] / args.steps) / HBM_PEAK_GBS, 4)},
     }
     lat_ticks, bpt, measured = q.hold_model()
     extra = {"hold_gate": {"latency_ticks": lat_ticks, "bytes_per_tick": bpt, "measured_on_this_device": measured,
